@@ -1,0 +1,108 @@
+/* C ABI of libqtip_hip.so: MI355X (gfx950) kernels for QTIP's quantized-linear
+ * inference path (HYB code: L=16, 9-bit tunable LUT, V=2, 16x16 trellis tiles,
+ * 2/3/4 bits per weight).
+ *
+ * Conventions for every launcher
+ *   - all pointers are DEVICE pointers on the current HIP device, plain C types;
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - asynchronous: the call enqueues work and returns; it never synchronises,
+ *     allocates, frees or queries device properties, so it may be recorded
+ *     into a HIP graph;
+ *   - returns 0 on success, a negative QTIP_E_* code for rejected arguments
+ *     (nothing was launched), or a positive hipError_t from the launch.  It
+ *     never terminates the process (the reference's launcher exits on error,
+ *     qtip-kernels/src/inference.h:10-18).
+ *
+ * Packed layout (`packed`): the reference's kernel packing, m*k*bits/8 bytes,
+ * bytes indexed [m/32][k/32][lane 32][kh 2][mh 2][bits] (produced by
+ * lib/algo/finetune.py:196-201, consumed by qtip-kernels/src/inference.cu:94-166).
+ * `tlut` is the raw tunable table, 512 x (fp16, fp16), 2 KiB.
+ */
+#ifndef QTIP_HIP_H
+#define QTIP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QTIP_OK 0
+#define QTIP_E_SHAPE (-1)     /* m % 32, k % 32, bits, batch or n out of range */
+#define QTIP_E_NULL (-2)      /* a required pointer is NULL */
+#define QTIP_E_ALIGN (-3)     /* a pointer is not 16-byte aligned */
+#define QTIP_E_WORKSPACE (-4) /* workspace smaller than qtip_matvec_workspace_bytes */
+#define QTIP_E_DTYPE (-5)     /* unknown dtype code */
+
+#define QTIP_F16 0
+#define QTIP_F32 1
+
+/* Library ABI version (bumped when a signature changes). */
+int qtip_abi_version(void);
+
+/* Text for a return code of any launcher below (static storage). */
+const char* qtip_error_string(int code);
+
+/* Dense decode of the kernel-packed stream: out[m][k] fp16, row-major.
+ * Replaces decode_compressed(L,S,R,V,m,k,compressed,expanded_lut)
+ * (lib/utils/kernel_decompress.py:4-55) and BitshiftLinear.get_hatW_kernel
+ * (lib/codebook/bitshift.py:383-387); takes the raw 512x2 table and applies
+ * the quantlut_sym expansion (lib/codebook/bitshift.py:72-80) on the fly.
+ * Bit-exact with the reference decode. */
+int qtip_decode(void* out_f16, const void* packed, const void* tlut,
+                int m, int k, int bits, void* stream);
+
+/* Bytes of scratch qtip_decompress_matvec wants for this shape (0 = none).
+ * Its first 64 KiB (arrival counters) must be zero before the first use; every
+ * call leaves them zero again, so one buffer can serve calls of any shape.
+ * Calls that share one scratch buffer must not overlap in time. */
+size_t qtip_matvec_workspace_bytes(int m, int k, int bits);
+
+/* bs=1 decompress + matvec: out[m] (fp32) = hatW[m][k] . x[k] (fp16), fp32
+ * accumulate, deterministic summation order, `out` fully overwritten.
+ * Replaces decompress_matvec_ptr<16,9,R,1,M,1,K>(float*, const uint32_t*,
+ * const half2*, const half2*, CUstream_st*) (qtip-kernels/src/inference.h:48-55,
+ * inference.cu:432-471) and the 64 pybind entry points
+ * decompress_matvec_16_9_{R}_1_{M}_1_{K} (qtip-kernels/src/wrapper.cpp:489-564).
+ * Shapes are run-time arguments: m % 32 == 0, k % 32 == 0, bits in {2,3,4}.
+ * `workspace` may be NULL (then the k dimension is never split across
+ * workgroups, which costs parallelism on small m). */
+int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16,
+                           const void* tlut, int m, int k, int bits,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* Batched decompress + GEMM on the matrix cores:
+ * out[batch][m] = x[batch][k] (fp16) . hatW[m][k]^T, fp32 accumulate.
+ * If round_f16 != 0 every result is rounded to fp16 and widened again, which
+ * is what the reference's fp16 GEMM output followed by .float() yields.
+ * Replaces BitshiftLinearKernelAG.forward = decode_compressed + input.half() @ hatW.T
+ * (lib/codebook/bitshift.py:476-489).  1 <= batch <= 65535. */
+int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16,
+                         const void* tlut, int m, int k, int bits, int batch,
+                         int round_f16, void* stream);
+
+/* Randomised Hadamard transform of `rows` vectors of length n = order * p
+ * (p a power of two, order 1 or a table order):
+ *   out[r][:] = post[:] * scale * (H_order (x) H_p) (pre[:] * in[r][:])
+ * with H_p the Sylvester (natural order) Walsh-Hadamard matrix.
+ *   in_dtype/out_dtype  QTIP_F16 or QTIP_F32
+ *   pre   fp16[n] or NULL (input sign vector SU)
+ *   post  fp32[n] or NULL (output scale vector SV)
+ *   had_bits  order*order sign bits, bit (i*order+j) of a little-endian
+ *             uint32 array set when H[i][j] == -1, already transposed by the
+ *             caller for the "Ut" form; ignored (may be NULL) when order == 1
+ *   in_parts  > 1: `in` holds in_parts arrays of rows*n elements that are
+ *             summed on load (split-k partial sums); normally 1.
+ * Replaces matmul_hadU_cuda / matmul_hadUt_cuda and the hadamard::hadamard
+ * op (lib/utils/matmul_had.py:92-119; third-party fast_hadamard_transform
+ * kernel + dense hadK matmul) together with the elementwise SU / SV / scale
+ * steps of BitshiftLinear.forward (lib/codebook/bitshift.py:428-441,469-472). */
+int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_parts,
+             int rows, int n, int order, const uint32_t* had_bits,
+             const void* pre_f16, const float* post_f32, float scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QTIP_HIP_H */

@@ -1,0 +1,230 @@
+"""BitshiftLinear on the HIP kernels: the drop-in for lib/codebook/bitshift.py.
+
+Kept from the reference: class names, constructor and forward signatures,
+attribute names (`cb`, `scale`, `internal_dtype`, `has_kernel`), tensor
+layouts and the cast points of the forward pass.  The quantiser side of
+`bitshift_codebook` (Viterbi, `quantize`, `update`) is not part of the
+inference path and raises NotImplementedError.
+"""
+import math
+
+import torch
+from torch import nn
+
+from .. import ops
+from ..utils.kernel_check import has_kernel as _has_kernel
+from ..utils.matmul_had import had_bits, matmul_hadU_cuda, matmul_hadUt_cuda
+from . import kdict, register_shape
+
+
+def quantlut_sym(tlut, L, nbits):
+    """HYB expansion of the tunable table to all 2**L states
+    (lib/codebook/bitshift.py:72-80): index bits 6..14 of s*(s+1) (for
+    nbits = 9), element 0 negated when bit 15 is set."""
+    with torch.no_grad():
+        s = torch.arange(1 << L, device=tlut.device)
+        p = (s + 1) * s
+        flip = 1 - ((p >> 15) & 1) * 2
+        idx = (p >> (16 - nbits - 1)) & ((1 << nbits) - 1)
+    lut = tlut[idx]
+    lut[:, 0] = lut[:, 0] * flip
+    return lut
+
+
+class bitshift_codebook(nn.Module):
+    """Inference part of the reference class (lib/codebook/bitshift.py:83-201):
+    holds the tunable table and its expansion; `recons` maps states to weights."""
+
+    def __init__(self, L=16, K=2, V=2, tlut_bits=16, decode_mode='lut', tlut=None):
+        super().__init__()
+        self.idx_dtype = torch.int32
+        self.opt_scale = 1
+        self.L, self.K, self.V = L, K, V
+        self.tlut_bits = tlut_bits
+        self.decode_mode = decode_mode
+        if decode_mode != 'quantlut_sym':
+            raise NotImplementedError(f"decode_mode {decode_mode!r}: only the HYB code 'quantlut_sym' is built")
+        if V != 2:
+            raise NotImplementedError("quantlut_sym needs V == 2")
+        if tlut is None:
+            # the reference fits a k-means table here (bitshift.py:147-168); a
+            # checkpoint always overwrites it, so start from a seeded Gaussian table
+            g = torch.Generator().manual_seed(0)
+            tlut = torch.randn(2**tlut_bits, V, generator=g)
+            tlut = (tlut / tlut.std(unbiased=False)) * 0.9682458365518543
+            self.register_buffer('tlut', tlut)
+            self.register_buffer('lut', quantlut_sym(self.tlut, L, tlut_bits).T.contiguous())
+        else:
+            self.tlut = tlut
+            self.recons_lut()
+        self.version = 0
+
+    def recons_lut(self):
+        self.lut = quantlut_sym(self.tlut, self.L, self.tlut_bits).T.contiguous()
+
+    def recons(self, encoded, **kwargs):
+        return self.lut[:, encoded.int().to(self.lut.device)].to(encoded.device)
+
+    def unpack_trellis(self, packed, T):
+        """Natural (non-kernel) packing -> (ntiles, T/V) states
+        (lib/codebook/bitshift.py:329-353), vectorised: state i is the 16-bit
+        window at bit offset i*K*V of the tile's circular bitstream."""
+        words = packed.view(torch.uint16).to(torch.int32).reshape(-1, T * self.K // 16)
+        nxt = torch.roll(words, -1, dims=1)
+        win = (words << 16) | nxt
+        kv = self.K * self.V
+        pos = torch.arange(T // self.V, device=packed.device) * kv
+        w_idx, off = pos // 16, pos % 16
+        return ((win[:, w_idx] >> (16 - off)) & 0xFFFF).to(torch.int32)
+
+    def quantize(self, *a, **k):
+        raise NotImplementedError("quantisation (Viterbi) is outside the inference path")
+
+    viterbi = update = quantize_seq = pack_trellis = quantize
+
+
+class BitshiftLinear(nn.Module):
+
+    def __init__(self, td_x, td_y, L, K, V, tlut_bits, decode_mode, dtype=torch.float16, tlut=None,
+                 has_kernel=False):
+        super().__init__()
+        self.td_x = td_x
+        self.td_y = td_y
+        self.V = V
+        self.cb = bitshift_codebook(L, K, V, tlut_bits, decode_mode, tlut=tlut)
+        self.internal_dtype = dtype
+        self.has_kernel = has_kernel
+        self.scale = 32
+        if has_kernel and not _has_kernel(decode_mode, L, K, V, tlut_bits, td_x, td_y):
+            raise ValueError("has_kernel=True for a configuration the kernels do not cover")
+
+    # -- dense weights -----------------------------------------------------
+    def get_hatW(self, unpacked_trellis, m, n):
+        """States in the natural packing -> (m, n) (lib/codebook/bitshift.py:378-381)."""
+        return self.cb.recons(unpacked_trellis).transpose(0, 1).transpose(1, 2).reshape(
+            m // self.td_x, n // self.td_y, self.td_x, self.td_y).transpose(1, 2).reshape(m, n)
+
+    def get_hatW_kernel(self, trellis, m, n):
+        """Kernel-packed trellis -> (m, n) fp16 on the HIP decode kernel
+        (lib/codebook/bitshift.py:383-387)."""
+        return ops.decode(trellis.reshape(-1), self._tlut16(trellis.device), m, n, self.cb.K)
+
+    def _tlut16(self, device):
+        t = self.cb.tlut
+        if t.dtype != torch.float16 or t.device != device or not t.is_contiguous():
+            t = t.to(device=device, dtype=torch.float16).contiguous()
+        return t
+
+    def cache_hatW(self, packed_trellis, had_left, had_right, K_left, K_right, m, n, rcp, tp_rank):
+        """Dense transformed weight for mode='train-fixW' (lib/codebook/bitshift.py:389-413)."""
+        if self.has_kernel:
+            hatW = self.get_hatW_kernel(packed_trellis, m, n)
+        else:
+            hatW = self.get_hatW(self.cb.unpack_trellis(packed_trellis, self.td_x * self.td_y), m, n)
+        hatW = hatW.float() / self.scale
+        if rcp == 1:
+            self.hatW = matmul_hadU_cuda(
+                matmul_hadU_cuda(hatW.reshape(tp_rank * m, n // tp_rank), had_left, K_left).reshape(m, n).T.contiguous(),
+                had_right, K_right).T.contiguous().to(self.internal_dtype)
+        elif rcp == 2:
+            self.hatW = matmul_hadU_cuda(
+                matmul_hadU_cuda(hatW, had_left, K_left).T.contiguous().reshape(tp_rank * n, m // tp_rank), had_right,
+                K_right).reshape(n, m).T.contiguous().to(self.internal_dtype)
+        else:
+            self.hatW = matmul_hadU_cuda(
+                matmul_hadU_cuda(hatW, had_left, K_left).T.contiguous(), had_right,
+                K_right).T.contiguous().to(self.internal_dtype)
+
+    # -- forward -------------------------------------------------------------
+    def forward(self, input, trellis, SU, SV, had_left, had_right, K_left, K_right, rcp, tp_rank,
+                mode='eval', **kwargs):
+        """y = (H_R [hatW fp16(H_L^T (x * SU) / 32)]) * (SV * 32), cast to input.dtype
+        (lib/codebook/bitshift.py:415-472).  Launches: RHT-in, matvec or GEMM, RHT-out."""
+        n, m = len(SU), len(SV)
+        if mode == 'train-fixW':
+            x = input.view(-1, n).to(torch.float32) * SU
+            x = (x.to(self.internal_dtype) @ self.hatW.T).float()
+            x = x.to(SV.device) * (SV * self.scale)
+            return x.view(*input.shape[:-1], m).to(input.dtype)
+        if mode not in ('eval', 'train-recons'):
+            raise NotImplementedError(f"mode {mode!r}")
+        if mode == 'train-recons':
+            self.cb.recons_lut()
+        rcp = int(rcp)
+        tp_rank = int(tp_rank)
+        dev = input.device
+        x = input.reshape(-1, n)
+        bs = x.shape[0]
+
+        # ---- input transform: fp16(H_L^T (x * SU) / sqrt(n) / 32)
+        fused_in = (rcp != 1 and SU.dtype == torch.float16 and x.dtype in (torch.float16, torch.float32))
+        if fused_in:
+            xt = ops.rht(x.contiguous(), order=K_left,
+                         had_bits=had_bits(had_left, K_left, True, dev) if K_left > 1 else None,
+                         pre=SU.contiguous(), scale=(n**-0.5) / self.scale, out_dtype=torch.float16)
+        else:
+            xf = x.to(torch.float32) * SU
+            if rcp == 1:
+                xf = xf.reshape(-1, n // tp_rank)
+            nn_ = xf.shape[-1]
+            xt = ops.rht(xf.contiguous(), order=K_left,
+                         had_bits=had_bits(had_left, K_left, True, dev) if K_left > 1 else None,
+                         scale=(nn_**-0.5) / self.scale, out_dtype=torch.float16).reshape(bs, n)
+
+        # ---- quantised matmul
+        if self.has_kernel:
+            tl = self._tlut16(dev)
+            if bs == 1:
+                key = (m, 1, n, self.cb.K)
+                wrapper = kdict.get(key) or register_shape(m, n, self.cb.K)
+                y = wrapper(trellis, xt, tl)
+            else:
+                y = ops.decompress_gemm(trellis.reshape(-1), xt, tl, m, n, self.cb.K, round_f16=True)
+        else:
+            st = trellis if mode != 'eval' else self.cb.unpack_trellis(trellis, self.td_x * self.td_y)
+            hatW = self.get_hatW(st, m, n)
+            y = (xt.to(hatW.dtype) @ hatW.T).float()
+
+        # ---- output transform: (H_R y / sqrt(m)) * SV * 32, cast
+        fused_out = (rcp != 2 and SV.dtype == torch.float32 and SV.device == dev
+                     and input.dtype in (torch.float16, torch.float32))
+        if fused_out:
+            out = ops.rht(y, order=K_right,
+                          had_bits=had_bits(had_right, K_right, False, dev) if K_right > 1 else None,
+                          post=SV.contiguous(), scale=(m**-0.5) * self.scale, out_dtype=input.dtype)
+        else:
+            yy = y.reshape(-1, m // tp_rank) if rcp == 2 else y
+            mm = yy.shape[-1]
+            yt = ops.rht(yy.contiguous(), order=K_right,
+                         had_bits=had_bits(had_right, K_right, False, dev) if K_right > 1 else None,
+                         scale=mm**-0.5, out_dtype=torch.float32).reshape(bs, m)
+            out = (yt.to(SV.device) * (SV * self.scale)).to(input.dtype)
+        return out.view(*input.shape[:-1], m)
+
+
+class BitshiftLinearKernelAG(torch.autograd.Function):
+    """x @ decode(trellis)^T with the weights re-decoded in backward
+    (lib/codebook/bitshift.py:476-505).  Forward uses the fused
+    decompress-GEMM; backward decodes to a dense matrix and uses a dense GEMM."""
+
+    @staticmethod
+    def forward(ctx, input, trellis, m, n, L, tlut_bits, K, V, lut):
+        from ..utils.kernel_decompress import tlut_from_expanded
+        tlut = tlut_from_expanded(lut.T)
+        ctx.save_for_backward(trellis, tlut)
+        ctx.shape = (m, n, K)
+        x = input.to(torch.float16).reshape(-1, n).contiguous()
+        if x.shape[0] == 1:
+            y = ops.decompress_matvec(trellis.reshape(-1), x.reshape(-1), tlut.reshape(-1), m, n, K).view(1, m)
+            y = y.to(torch.float16)
+        else:
+            y = ops.decompress_gemm(trellis.reshape(-1), x, tlut.reshape(-1), m, n, K, round_f16=True).to(torch.float16)
+        return y.view(*input.shape[:-1], m)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        trellis, tlut = ctx.saved_tensors
+        m, n, K = ctx.shape
+        hatW = ops.decode(trellis.reshape(-1), tlut.reshape(-1), m, n, K)
+        grad_input = grad_output.to(hatW.dtype) @ hatW
+        return grad_input, None, None, None, None, None, None, None, None

@@ -1,0 +1,175 @@
+// Device-side building blocks shared by the decode, matvec and GEMM kernels.
+//
+// Lane mapping (all bit widths K = 2,3,4).  The packed stream is an array
+// [m/32][k/32][ref lane 32][kh 2][mh 2][K bytes]: one 2x2 block of 16x16 tiles
+// is 128*K contiguous bytes and "ref lane" l owns 4*K of them (one K-byte
+// chunk of each of the four tiles).  A chunk decodes only together with the
+// leading 16 bits of ref lane (l+1) mod 32's chunk of the same tile.
+//
+// A 64-wide wavefront reads four consecutive 2x2 blocks ("wave-load",
+// 512*K bytes).  Lane = 16*g + a takes block g and the two ref lanes 2a and
+// 2a+1, i.e. 8*K contiguous bytes.  Ref lane 2a finds its successor in the
+// same lane's registers; ref lane 2a+1 needs lane a+1's first chunk, and the
+// ring closes inside the 16-lane DPP row (row_ror:15), so the neighbour
+// exchange never leaves the VALU.
+//
+// Per wave-load a lane decodes 32 states = 64 weights:
+//   rows    32*rb + 16*mh + 8*rh + a/2          (mh, rh in {0,1})
+//   columns 32*kb + 16*kh + 8*jh + 4*(a%2) + {0,1 (ref A), 2,3 (ref B)}
+// with tile t = 2*kh + mh inside the ref lane's bytes and state j = 2*jh + rh
+// inside the chunk.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qtip {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// LDS weight table: 1024 entries (9 index bits + the sign bit of the hash as
+// a tenth), each replicated 16 times so that a lane reads replica (lane % 16).
+// Entry e sits at byte e*64, which is exactly bits 6..15 of the hash value.
+constexpr int kLutEntries = 1024;
+constexpr int kLutBytes = kLutEntries * 64;
+
+// Fill the table from the raw 512 x (fp16,fp16) tunable LUT.  Entry
+// e = sign*512 + q holds tlut[q] with element 0 (the low half) negated when
+// sign is set: the quantlut_sym rule.
+__device__ __forceinline__ void build_lut(uint32_t* lut, const uint32_t* __restrict__ tlut,
+                                          int tid, int nthreads) {
+  for (int e = tid; e < kLutEntries; e += nthreads) {
+    uint32_t w = tlut[e & 511] ^ ((uint32_t)(e >> 9) << 15);
+    u32x4 v = {w, w, w, w};
+    u32x4* dst = reinterpret_cast<u32x4*>(lut + e * 16);
+    dst[0] = v;
+    dst[1] = v;
+    dst[2] = v;
+    dst[3] = v;
+  }
+}
+
+template <int K>
+struct LaneData {
+  uint32_t d[2 * K];  // ref lane A = d[0..K), ref lane B = d[K..2K)
+};
+
+// Streaming load of a lane's 8*K bytes (read once, keep out of the caches'
+// way with the non-temporal hint).
+template <int K>
+__device__ __forceinline__ LaneData<K> load_lane(const uint8_t* __restrict__ p) {
+  LaneData<K> r;
+  if constexpr (K == 3) {
+    const u32x2* q = reinterpret_cast<const u32x2*>(p);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      u32x2 v = __builtin_nontemporal_load(q + i);
+      r.d[2 * i] = v[0];
+      r.d[2 * i + 1] = v[1];
+    }
+  } else {
+    const u32x4* q = reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int i = 0; i < K / 2; ++i) {
+      u32x4 v = __builtin_nontemporal_load(q + i);
+      r.d[4 * i] = v[0];
+      r.d[4 * i + 1] = v[1];
+      r.d[4 * i + 2] = v[2];
+      r.d[4 * i + 3] = v[3];
+    }
+  }
+  return r;
+}
+
+// Chunk of tile t of one ref lane (e = that ref lane's K dwords) as the
+// big-endian integer of its 8*K stream bits.
+template <int K>
+__device__ __forceinline__ uint32_t chunk(const uint32_t* e, int t) {
+  if constexpr (K == 2) {
+    return (t & 1) ? (e[t >> 1] >> 16) : (e[t >> 1] & 0xFFFFu);
+  } else if constexpr (K == 3) {
+    switch (t) {
+      case 0: return e[0] & 0xFFFFFFu;
+      case 1: return (e[0] >> 24) | ((e[1] & 0xFFFFu) << 8);
+      case 2: return (e[1] >> 16) | ((e[2] & 0xFFu) << 16);
+      default: return e[2] >> 8;
+    }
+  } else {
+    return e[t];
+  }
+}
+
+// value of lane (a+1) mod 16 of the same 16-lane row
+__device__ __forceinline__ uint32_t from_next_lane16(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x12F /* row_ror:15 */, 0xF, 0xF, false);
+}
+
+// All 32 states of a lane's wave-load: st[R][t][j], R = ref lane (A,B),
+// t = tile 2*kh+mh, j = state inside the chunk.  Only the low 16 bits of each
+// value are meaningful; higher bits hold leftovers of the window and are
+// harmless because the hash uses the low 16 bits of its result only.
+template <int K>
+__device__ __forceinline__ void lane_states(const LaneData<K>& ld, uint32_t st[2][4][4]) {
+  uint32_t own[2][4], top[2][4];
+#pragma unroll
+  for (int R = 0; R < 2; ++R)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      own[R][t] = chunk<K>(&ld.d[R * K], t);
+      top[R][t] = own[R][t] >> (8 * K - 16);
+    }
+  // what the previous lane's ref B needs from this lane's ref A
+  uint32_t s01, s23;
+  if constexpr (K == 2) {
+    s01 = ld.d[0];
+    s23 = ld.d[1];
+  } else {
+    s01 = top[0][0] | (top[0][1] << 16);
+    s23 = top[0][2] | (top[0][3] << 16);
+  }
+  const uint32_t r01 = from_next_lane16(s01);
+  const uint32_t r23 = from_next_lane16(s23);
+  uint32_t nxt[2][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) nxt[0][t] = top[1][t];
+  nxt[1][0] = r01 & 0xFFFFu;
+  nxt[1][1] = r01 >> 16;
+  nxt[1][2] = r23 & 0xFFFFu;
+  nxt[1][3] = r23 >> 16;
+#pragma unroll
+  for (int R = 0; R < 2; ++R)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint32_t o = own[R][t];
+      const uint32_t v = (o << 16) | nxt[R][t];  // low 32 bits of chunk || next16
+      if constexpr (K == 2) {
+        st[R][t][0] = o;
+        st[R][t][1] = v >> 12;
+        st[R][t][2] = v >> 8;
+        st[R][t][3] = v >> 4;
+      } else if constexpr (K == 3) {
+        st[R][t][0] = o >> 8;
+        st[R][t][1] = o >> 2;
+        st[R][t][2] = v >> 12;
+        st[R][t][3] = v >> 6;
+      } else {
+        st[R][t][0] = o >> 16;
+        st[R][t][1] = o >> 8;
+        st[R][t][2] = o;
+        st[R][t][3] = v >> 8;
+      }
+    }
+}
+
+// HYB lookup: p = s*(s+1); bits 6..15 of p address the sign-folded table.
+__device__ __forceinline__ uint32_t lut_lookup(const uint32_t* lut, uint32_t s, uint32_t slot4) {
+  const uint32_t p = __umul24(s, s) + s;
+  const uint32_t addr = (p & 0xFFC0u) | slot4;
+  return *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(lut) + addr);
+}
+
+}  // namespace qtip

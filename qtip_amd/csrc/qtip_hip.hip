@@ -1,0 +1,678 @@
+// libqtip_hip.so: gfx950 kernels and C ABI for QTIP's quantized-linear
+// inference path.  Declarations and the reference interfaces each entry
+// point replaces are in include/qtip_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qtip_hip.h"
+#include "qtip_device.h"
+
+using namespace qtip;
+
+namespace {
+
+constexpr int kThreads = 1024;  // 16 waves per workgroup, one workgroup per CU
+constexpr int kWaves = kThreads / 64;
+constexpr int kMaxSplit = 16;
+constexpr size_t kCounterBytes = 65536;  // arrival counters at the start of the matvec workspace
+
+__device__ __forceinline__ float dpp_xor1(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1 /* quad_perm 1,0,3,2 */,
+                                         0xF, 0xF, false));
+}
+__device__ __forceinline__ float swz_xor16(float v) {
+  return __builtin_bit_cast(float,
+                            __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+__device__ __forceinline__ float xor32(float v) {
+  uint32_t u = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // r[0]: lanes 0-31 keep their value, lanes 32-63 receive lanes 0-31;
+  // r[1]: lanes 0-31 receive lanes 32-63, lanes 32-63 keep theirs.
+  const bool upper = (threadIdx.x & 32) != 0;
+  return __builtin_bit_cast(float, upper ? r[0] : r[1]);
+}
+
+// ---------------------------------------------------------------------------
+// decode: packed stream -> dense fp16 (m, k)
+// ---------------------------------------------------------------------------
+template <int K>
+__global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restrict__ out,
+                                                             const uint8_t* __restrict__ packed,
+                                                             const uint32_t* __restrict__ tlut,
+                                                             int m, int k) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+  build_lut(lut, tlut, threadIdx.x, kThreads);
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int a = lane & 15, g = lane >> 4;
+  const uint32_t slot4 = (uint32_t)a << 2;
+  const int nkb = k >> 5;
+  const int nwl = (nkb + 3) >> 2;
+  const long total = (long)(m >> 5) * nwl;  // wave-loads in the matrix
+  const size_t rb_bytes = (size_t)nkb * 128 * K;
+  for (long w = (long)blockIdx.x * kWaves + wave; w < total; w += (long)gridDim.x * kWaves) {
+    const int rb = (int)(w / nwl), wl = (int)(w - (long)rb * nwl);
+    const int kb = 4 * wl + g;
+    if (kb >= nkb) continue;
+    const LaneData<K> ld =
+        load_lane<K>(packed + (size_t)rb * rb_bytes + (size_t)kb * 128 * K + a * 8 * K);
+    uint32_t st[2][4][4];
+    lane_states<K>(ld, st);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int kh = t >> 1, mh = t & 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int jh = j >> 1, rh = j & 1;
+        u32x2 v;
+        v[0] = lut_lookup(lut, st[0][t][j], slot4);
+        v[1] = lut_lookup(lut, st[1][t][j], slot4);
+        const size_t row = (size_t)rb * 32 + 16 * mh + 8 * rh + (a >> 1);
+        const size_t col = (size_t)kb * 32 + 16 * kh + 8 * jh + 4 * (a & 1);
+        *reinterpret_cast<u32x2*>(out + row * k + col) = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// decompress + matvec
+// ---------------------------------------------------------------------------
+template <int K>
+__device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld,
+                                                  const uint16_t* __restrict__ xp,
+                                                  const uint32_t* lut, uint32_t slot4,
+                                                  float acc[4]) {
+  // x for columns 8*q + 4*(a%2) + {0..3}, q = 2*kh + jh
+  u32x2 xv[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) xv[q] = *reinterpret_cast<const u32x2*>(xp + 8 * q);
+  uint32_t st[2][4][4];
+  lane_states<K>(ld, st);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int kh = t >> 1, mh = t & 1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int jh = j >> 1, rh = j & 1;
+#pragma unroll
+      for (int R = 0; R < 2; ++R) {
+        const uint32_t w = lut_lookup(lut, st[R][t][j], slot4);
+        // (copy the vector element to a scalar first: bit_cast applied directly
+        // to a vector-element lvalue reads element 0)
+        const uint32_t xr = xv[2 * kh + jh][R];
+        acc[2 * mh + rh] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w),
+                                                  __builtin_bit_cast(half2_t, xr),
+                                                  acc[2 * mh + rh], false);
+      }
+    }
+  }
+}
+
+// Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup share
+// a unit's wave-loads round-robin, reduce through LDS in a fixed order and
+// either store the 32 results (S == 1) or publish a partial row block; the
+// last workgroup to arrive for a row block adds the S partials in order
+// 0..S-1, so the result does not depend on scheduling.
+template <int K, int DEPTH>
+__global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
+    float* __restrict__ out, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut, int m, int k, int S, float* ws, unsigned* counters) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+  float* part = reinterpret_cast<float*>(smem + kLutBytes);  // [kWaves][32]
+  __shared__ int s_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int a = lane & 15, g = lane >> 4;
+  const uint32_t slot4 = (uint32_t)a << 2;
+  const int nkb = k >> 5;
+  const int nwl = (nkb + 3) >> 2;
+  const size_t rb_bytes = (size_t)nkb * 128 * K;
+  const int units = (m >> 5) * S;
+  const uint16_t* xlane = x + 4 * (a & 1) + 32 * g;
+  constexpr int WL_BYTES = 512 * K;
+
+  build_lut(lut, tlut, tid, kThreads);
+  __syncthreads();
+
+  for (int u = blockIdx.x; u < units; u += gridDim.x) {
+    const int rb = u / S, s = u - rb * S;
+    const int wl0 = (int)((long)s * nwl / S), wl1 = (int)((long)(s + 1) * nwl / S);
+    const uint8_t* base = packed + (size_t)rb * rb_bytes + (size_t)g * 128 * K + a * 8 * K;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+
+    LaneData<K> buf[DEPTH];
+    int wl = wl0 + wave;
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int w = wl + d * kWaves;
+      if (w < wl1 && 4 * w + g < nkb) buf[d] = load_lane<K>(base + (size_t)w * WL_BYTES);
+    }
+    for (; wl < wl1; wl += DEPTH * kWaves) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int w = wl + d * kWaves;
+        if (w < wl1) {
+          const LaneData<K> cur = buf[d];
+          const int wn = w + DEPTH * kWaves;
+          if (wn < wl1 && 4 * wn + g < nkb) buf[d] = load_lane<K>(base + (size_t)wn * WL_BYTES);
+          if (4 * w + g < nkb) matvec_accumulate<K>(cur, xlane + (size_t)w * 128, lut, slot4, acc);
+        }
+      }
+    }
+
+    // lanes sharing a row differ in lane bits 0 (column half), 4 and 5 (block)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = acc[i];
+      v += dpp_xor1(v);
+      v += swz_xor16(v);
+      v += xor32(v);
+      if (g == 0 && (a & 1) == 0) part[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
+    }
+    __syncthreads();
+    if (tid < 32) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) sum += part[w * 32 + tid];
+      if (S == 1) {
+        out[rb * 32 + tid] = sum;
+      } else {
+        __hip_atomic_store(ws + (size_t)s * m + rb * 32 + tid, sum, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (S > 1) {
+      __threadfence();
+      __syncthreads();
+      if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(counters + rb, 1u, __ATOMIC_ACQ_REL,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == (unsigned)(S - 1));
+      }
+      __syncthreads();
+      if (s_last) {
+        __threadfence();
+        if (tid < 32) {
+          float sum = 0.f;
+          for (int s2 = 0; s2 < S; ++s2)
+            sum += __hip_atomic_load(ws + (size_t)s2 * m + rb * 32 + tid, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+          out[rb * 32 + tid] = sum;
+        }
+        if (tid == 0)
+          __hip_atomic_store(counters + rb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// batched decompress -> LDS -> fp16 MFMA GEMM
+// ---------------------------------------------------------------------------
+constexpr int kGemmThreads = 512;
+constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kStageStride = 128 + 8;                  // halfs per staged row (padding vs banks)
+constexpr int kStageHalfs = 32 * kStageStride;         // one wave's 32 x 128 tile
+constexpr int kStageBytes = kStageHalfs * 2;           // 8704
+
+// out[b][row] for b < batch.  NB = number of 16-wide batch tiles per pass.
+template <int K, int NB>
+__global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
+    float* __restrict__ out, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+  uint8_t* stage_all = smem + kLutBytes;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int a = lane & 15, g = lane >> 4;
+  const uint32_t slot4 = (uint32_t)a << 2;
+  const int nkb = k >> 5;
+  const int nwl = (nkb + 3) >> 2;
+  const size_t rb_bytes = (size_t)nkb * 128 * K;
+  const int nrb = m >> 5;
+  constexpr int WL_BYTES = 512 * K;
+  uint16_t* stage = reinterpret_cast<uint16_t*>(stage_all + wave * kStageBytes);
+  float* red = reinterpret_cast<float*>(stage_all);  // reused after the k loop
+
+  build_lut(lut, tlut, tid, kGemmThreads);
+  __syncthreads();
+
+  const int row16 = lane & 15, kgrp = lane >> 4;  // MFMA operand coordinates
+
+  for (int rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const uint8_t* base = packed + (size_t)rb * rb_bytes + (size_t)g * 128 * K + a * 8 * K;
+    float4_t acc[2][NB];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[mt][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int wl = wave; wl < nwl; wl += kGemmWaves) {
+      const int kb = 4 * wl + g;
+      const bool active = kb < nkb;
+      uint32_t st[2][4][4];
+      if (active) {
+        const LaneData<K> ld = load_lane<K>(base + (size_t)wl * WL_BYTES);
+        lane_states<K>(ld, st);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int kh = t >> 1, mh = t & 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int jh = j >> 1, rh = j & 1;
+          u32x2 v = {0u, 0u};
+          if (active) {
+            v[0] = lut_lookup(lut, st[0][t][j], slot4);
+            v[1] = lut_lookup(lut, st[1][t][j], slot4);
+          }
+          const int row = 16 * mh + 8 * rh + (a >> 1);
+          const int col = 32 * g + 16 * kh + 8 * jh + 4 * (a & 1);
+          *reinterpret_cast<u32x2*>(stage + row * kStageStride + col) = v;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const size_t kcol0 = (size_t)wl * 128;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int kc = 32 * ks + 8 * kgrp;
+        half8_t bfrag[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int b = 16 * nb + row16;
+          u32x4 raw = {0u, 0u, 0u, 0u};
+          if (b < batch && kcol0 + kc < (size_t)k)
+            raw = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + kcol0 + kc);
+          bfrag[nb] = __builtin_bit_cast(half8_t, raw);
+        }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const half8_t afrag = *reinterpret_cast<const half8_t*>(
+              stage + (16 * mt + row16) * kStageStride + kc);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            acc[mt][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag[nb], acc[mt][nb], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+
+    // cross-wave reduction: red[wave][row 32][col 16*NB]
+    __syncthreads();
+    constexpr int NC = 16 * NB;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          red[(wave * 32 + 16 * mt + 4 * kgrp + i) * NC + 16 * nb + row16] = acc[mt][nb][i];
+    __syncthreads();
+    for (int e = tid; e < 32 * NC; e += kGemmThreads) {
+      const int b = e >> 5, row = e & 31;  // consecutive threads -> consecutive rows of out
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kGemmWaves; ++w) sum += red[(w * 32 + row) * NC + b];
+      if (round_f16) sum = (float)(_Float16)sum;
+      if (b < batch) out[(size_t)b * m + rb * 32 + row] = sum;
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// randomised Hadamard transform
+// ---------------------------------------------------------------------------
+constexpr int kRhtThreads = 256;
+constexpr int kRhtMaxP = 8192;
+
+template <typename T>
+__device__ __forceinline__ float load_as_float(const T* p, size_t i);
+template <>
+__device__ __forceinline__ float load_as_float<float>(const float* p, size_t i) {
+  return p[i];
+}
+template <>
+__device__ __forceinline__ float load_as_float<_Float16>(const _Float16* p, size_t i) {
+  return (float)p[i];
+}
+
+// grid (order_total, rows).  Workgroup (i, r) produces the p outputs
+// out[r][i*p .. i*p+p): first the order-wide mix z[c] = sum_j H[i][j] v[j*p+c]
+// (H = table bits, or the Sylvester sign parity(i & j) for the power-of-two
+// pre-split), then a p-point Walsh-Hadamard transform of z in LDS.
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(kRhtThreads) void rht_kernel(
+    TOut* __restrict__ out, const TIn* __restrict__ in, int in_parts, size_t part_stride, int n,
+    int order, int p, int sylvester, const uint32_t* __restrict__ had_bits,
+    const _Float16* __restrict__ pre, const float* __restrict__ post, float scale) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  float* buf = reinterpret_cast<float*>(smem);  // [p]
+  float* red = buf + p;                         // [kRhtThreads] when p < kRhtThreads
+  const int tid = threadIdx.x;
+  const int i = blockIdx.x;
+  const size_t r = blockIdx.y;
+  const TIn* src = in + r * (size_t)n;
+
+  const int C = p < kRhtThreads ? p : kRhtThreads;  // columns per pass
+  const int JG = kRhtThreads / C;                   // j groups working on one column
+  const int c_in = tid % C, jg = tid / C;
+  for (int c0 = 0; c0 < p; c0 += C) {
+    const int c = c0 + c_in;
+    float z = 0.f;
+    for (int j = jg; j < order; j += JG) {
+      const size_t idx = (size_t)j * p + c;
+      float v = load_as_float<TIn>(src, idx);
+      for (int q = 1; q < in_parts; ++q) v += load_as_float<TIn>(src + q * part_stride, idx);
+      if (pre) v *= (float)pre[idx];
+      int neg;
+      if (sylvester) {
+        neg = __builtin_popcount(i & j) & 1;
+      } else {
+        const unsigned bit = (unsigned)i * order + j;
+        neg = (had_bits[bit >> 5] >> (bit & 31)) & 1;
+      }
+      z += neg ? -v : v;
+    }
+    if (JG > 1) {
+      red[tid] = z;
+      __syncthreads();
+      if (jg == 0) {
+        for (int q = 1; q < JG; ++q) z += red[q * C + c_in];
+        buf[c] = z;
+      }
+      __syncthreads();
+    } else {
+      buf[c] = z;
+    }
+  }
+  __syncthreads();
+  for (int h = 1; h < p; h <<= 1) {
+    for (int b = tid; b < (p >> 1); b += kRhtThreads) {
+      const int lo = ((b / h) * 2 * h) + (b % h);
+      const float u = buf[lo], w = buf[lo + h];
+      buf[lo] = u + w;
+      buf[lo + h] = u - w;
+    }
+    __syncthreads();
+  }
+  for (int c = tid; c < p; c += kRhtThreads) {
+    const size_t idx = (size_t)i * p + c;
+    float v = buf[c] * scale;
+    if (post) v *= post[idx];
+    out[r * (size_t)n + idx] = (TOut)v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct DeviceInfo {
+  int cus = 0;
+  bool ok = false;
+};
+
+// One-time per-process set-up (CU count, LDS opt-in).  Runs on the first call
+// of any launcher; callers that record HIP graphs make one eager call first.
+DeviceInfo& device_info() {
+  static DeviceInfo info = [] {
+    DeviceInfo d;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return d;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      return d;
+    d.cus = cus > 0 ? cus : 256;
+    d.ok = true;
+    return d;
+  }();
+  return info;
+}
+
+template <typename F>
+hipError_t allow_lds(F* fn, size_t bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+constexpr size_t kMatvecLds = kLutBytes + kWaves * 32 * sizeof(float);
+constexpr size_t kGemmLds = kLutBytes + kGemmWaves * kStageBytes;
+
+hipError_t setup_once() {
+  static hipError_t status = [] {
+    hipError_t e;
+#define QTIP_ALLOW(fn, bytes) \
+  if ((e = allow_lds(fn, bytes)) != hipSuccess) return e;
+    QTIP_ALLOW((decode_kernel<2>), kLutBytes)
+    QTIP_ALLOW((decode_kernel<3>), kLutBytes)
+    QTIP_ALLOW((decode_kernel<4>), kLutBytes)
+    QTIP_ALLOW((matvec_kernel<2, 4>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<3, 3>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<4, 2>), kMatvecLds)
+    QTIP_ALLOW((gemm_kernel<2, 1>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 2>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 4>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 1>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 2>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 4>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 1>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 2>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 4>), kGemmLds)
+#undef QTIP_ALLOW
+    return hipSuccess;
+  }();
+  return status;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_common(const void* a, const void* b, const void* c, const void* d, int m, int k,
+                 int bits) {
+  if (!a || !b || !c || !d) return QTIP_E_NULL;
+  if (bits < 2 || bits > 4) return QTIP_E_SHAPE;
+  if (m <= 0 || k <= 0 || (m & 31) || (k & 31)) return QTIP_E_SHAPE;
+  if ((long)m * k > (1L << 40)) return QTIP_E_SHAPE;
+  return QTIP_OK;
+}
+
+// k split so that (m/32)*S units fill the machine evenly
+int choose_split(int m, int k, int bits, int cus) {
+  const int nrb = m >> 5;
+  const int nwl = ((k >> 5) + 3) >> 2;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int S = 1; S <= kMaxSplit; S *= 2) {
+    if (nwl / S < kWaves && S > 1) break;  // keep at least one wave-load per wave
+    const long units = (long)nrb * S;
+    const long rounds = (units + cus - 1) / cus;
+    // cost: rounds * (unit bytes + fixed per-unit overhead expressed in bytes)
+    const double unit_bytes = (double)nwl / S * 512.0 * bits;
+    const double cost = rounds * (unit_bytes + 12288.0 + (S > 1 ? 4096.0 : 0.0));
+    if (cost < best_cost * 0.97) {
+      best_cost = cost;
+      best = S;
+    }
+  }
+  return best;
+}
+
+}  // namespace
+
+extern "C" {
+
+int qtip_abi_version(void) { return 1; }
+
+const char* qtip_error_string(int code) {
+  switch (code) {
+    case QTIP_OK: return "ok";
+    case QTIP_E_SHAPE: return "qtip: unsupported shape (need m % 32 == 0, k % 32 == 0, bits in 2..4, sizes in range)";
+    case QTIP_E_NULL: return "qtip: null pointer argument";
+    case QTIP_E_ALIGN: return "qtip: pointer not 16-byte aligned";
+    case QTIP_E_WORKSPACE: return "qtip: workspace too small";
+    case QTIP_E_DTYPE: return "qtip: unknown dtype code";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "qtip: unknown error";
+  }
+}
+
+int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int k, int bits,
+                void* stream) {
+  int rc = check_common(out_f16, packed, tlut, tlut, m, k, bits);
+  if (rc) return rc;
+  if (!aligned16(out_f16) || !aligned16(packed) || (reinterpret_cast<uintptr_t>(tlut) & 3u))
+    return QTIP_E_ALIGN;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return (int)hipErrorInvalidDevice;
+  hipError_t e = setup_once();
+  if (e != hipSuccess) return (int)e;
+  const long total = (long)(m >> 5) * (((k >> 5) + 3) >> 2);
+  long want = (total + kWaves - 1) / kWaves;
+  const int grid = (int)(want < di.cus ? want : di.cus);
+  hipStream_t st = (hipStream_t)stream;
+  auto* o = (uint16_t*)out_f16;
+  auto* p = (const uint8_t*)packed;
+  auto* t = (const uint32_t*)tlut;
+  switch (bits) {
+    case 2: decode_kernel<2><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
+    case 3: decode_kernel<3><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
+    default: decode_kernel<4><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
+  }
+  return (int)hipGetLastError();
+}
+
+size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
+  (void)k;
+  (void)bits;
+  if (m <= 0) return 0;
+  // fixed-size block of arrival counters (one per 32-row block; the only part
+  // that must stay zero between calls) followed by kMaxSplit partial vectors
+  return kCounterBytes + (size_t)kMaxSplit * m * sizeof(float);
+}
+
+int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,
+                           int m, int k, int bits, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
+  if (rc) return rc;
+  if (!aligned16(packed) || (reinterpret_cast<uintptr_t>(x_f16) & 7u) ||
+      (reinterpret_cast<uintptr_t>(tlut) & 3u) || (reinterpret_cast<uintptr_t>(out) & 3u))
+    return QTIP_E_ALIGN;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return (int)hipErrorInvalidDevice;
+  hipError_t e = setup_once();
+  if (e != hipSuccess) return (int)e;
+  int S = 1;
+  float* ws = nullptr;
+  unsigned* counters = nullptr;
+  if (workspace) {
+    if (workspace_bytes < qtip_matvec_workspace_bytes(m, k, bits)) return QTIP_E_WORKSPACE;
+    if (!aligned16(workspace)) return QTIP_E_ALIGN;
+    S = choose_split(m, k, bits, di.cus);
+    if ((size_t)(m >> 5) * sizeof(unsigned) > kCounterBytes) return QTIP_E_SHAPE;
+    counters = (unsigned*)workspace;
+    ws = (float*)((uint8_t*)workspace + kCounterBytes);
+  }
+  const long units = (long)(m >> 5) * S;
+  const int grid = (int)(units < di.cus ? units : di.cus);
+  hipStream_t st = (hipStream_t)stream;
+  auto* p = (const uint8_t*)packed;
+  auto* xx = (const uint16_t*)x_f16;
+  auto* t = (const uint32_t*)tlut;
+  switch (bits) {
+    case 2: matvec_kernel<2, 4><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
+    case 3: matvec_kernel<3, 3><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
+    default: matvec_kernel<4, 2><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
+  }
+  return (int)hipGetLastError();
+}
+
+int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, const void* tlut,
+                         int m, int k, int bits, int batch, int round_f16, void* stream) {
+  int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
+  if (rc) return rc;
+  if (batch < 1 || batch > 65535) return QTIP_E_SHAPE;
+  if (!aligned16(packed) || !aligned16(x_f16) || (reinterpret_cast<uintptr_t>(tlut) & 3u) ||
+      (reinterpret_cast<uintptr_t>(out) & 3u))
+    return QTIP_E_ALIGN;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return (int)hipErrorInvalidDevice;
+  hipError_t e = setup_once();
+  if (e != hipSuccess) return (int)e;
+  const int nrb = m >> 5;
+  const int grid = nrb < di.cus ? nrb : di.cus;
+  hipStream_t st = (hipStream_t)stream;
+  auto* p = (const uint8_t*)packed;
+  auto* t = (const uint32_t*)tlut;
+  // batch handled in passes of at most 64 rows
+  for (int b0 = 0; b0 < batch; b0 += 64) {
+    const int nb = batch - b0 < 64 ? batch - b0 : 64;
+    float* o = out + (size_t)b0 * m;
+    const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
+#define QTIP_GEMM(KB, NBT) \
+  gemm_kernel<KB, NBT><<<grid, kGemmThreads, kGemmLds, st>>>(o, p, xx, t, m, k, nb, round_f16)
+#define QTIP_GEMM_K(KB)            \
+  if (nb <= 16) QTIP_GEMM(KB, 1);  \
+  else if (nb <= 32) QTIP_GEMM(KB, 2); \
+  else QTIP_GEMM(KB, 4);
+    switch (bits) {
+      case 2: QTIP_GEMM_K(2) break;
+      case 3: QTIP_GEMM_K(3) break;
+      default: QTIP_GEMM_K(4) break;
+    }
+#undef QTIP_GEMM_K
+#undef QTIP_GEMM
+    hipError_t le = hipGetLastError();
+    if (le != hipSuccess) return (int)le;
+  }
+  return QTIP_OK;
+}
+
+int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
+             int order, const uint32_t* had_bits, const void* pre_f16, const float* post_f32,
+             float scale, void* stream) {
+  if (!out || !in) return QTIP_E_NULL;
+  if (rows < 1 || rows > 65535 || n < 1 || order < 1 || in_parts < 1 || in_parts > kMaxSplit)
+    return QTIP_E_SHAPE;
+  if (n % order) return QTIP_E_SHAPE;
+  int p = n / order;
+  if (p & (p - 1)) return QTIP_E_SHAPE;
+  if (order > 1 && !had_bits) return QTIP_E_NULL;
+  if ((unsigned)out_dtype > 1u || (unsigned)in_dtype > 1u) return QTIP_E_DTYPE;
+  int sylvester = 0, total_order = order;
+  if (order == 1) {
+    // split a power-of-two size as H_A (x) H_p with a small Sylvester factor
+    // A so that more than one workgroup works on a vector
+    sylvester = 1;
+    int A = 1;
+    while (A < 32 && p / 2 >= 256 && (A < 16 || p / 2 >= 512)) {
+      A *= 2;
+      p /= 2;
+    }
+    total_order = A;
+  }
+  if (p > kRhtMaxP) return QTIP_E_SHAPE;
+  const size_t lds = (size_t)p * sizeof(float) + (p < kRhtThreads ? kRhtThreads * sizeof(float) : 0);
+  dim3 grid(total_order, rows);
+  hipStream_t st = (hipStream_t)stream;
+  const size_t part_stride = (size_t)rows * n;
+  const _Float16* pre = (const _Float16*)pre_f16;
+#define QTIP_RHT(TI, TO)                                                                      \
+  rht_kernel<TI, TO><<<grid, kRhtThreads, lds, st>>>((TO*)out, (const TI*)in, in_parts,        \
+                                                     part_stride, n, total_order, p, sylvester, \
+                                                     had_bits, pre, post_f32, scale)
+  if (in_dtype == QTIP_F16 && out_dtype == QTIP_F16) QTIP_RHT(_Float16, _Float16);
+  else if (in_dtype == QTIP_F16 && out_dtype == QTIP_F32) QTIP_RHT(_Float16, float);
+  else if (in_dtype == QTIP_F32 && out_dtype == QTIP_F16) QTIP_RHT(float, _Float16);
+  else QTIP_RHT(float, float);
+#undef QTIP_RHT
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,0 +1,279 @@
+"""GPU: parity of the HIP kernels (called through the C ABI via ctypes) with the
+CPU oracle.  Decoded weights must be bit-exact; matvec / GEMM / layer outputs
+must meet max-rel <= 1e-2 and mean-rel <= 1e-3 (relative to the largest /
+mean magnitude of the oracle's output), the tolerance stated for the path."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import qtip_oracle as O
+from synth import make_layer
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL = 1e-2
+MEAN_REL = 1e-3
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_errors(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    d = np.abs(got - ref)
+    return d.max() / np.abs(ref).max(), d.mean() / np.abs(ref).mean()
+
+
+def assert_close(got, ref, max_rel=MAX_REL, mean_rel=MEAN_REL):
+    mx, mn = rel_errors(got, ref)
+    assert mx <= max_rel and mn <= mean_rel, (mx, mn)
+
+
+SMALL = [(32, 32), (64, 96), (256, 256), (96, 416), (1024, 4096 + 32)]
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("shape", SMALL)
+def test_decode_bit_exact(K, shape):
+    from qtip_amd import ops
+    m, k = shape
+    L = make_layer(m, k, K, seed=m + k + K)
+    got = ops.decode(dev(L["packed"]), dev(L["tlut"]), m, k, K).cpu().numpy()
+    ref = c_oracle.decode(L["packed"], L["tlut"], m, k, K)
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+def test_decode_bit_exact_4096(K):
+    from qtip_amd import ops
+    m = k = 4096
+    L = make_layer(m, k, K, seed=K)
+    got = ops.decode(dev(L["packed"]), dev(L["tlut"]), m, k, K).cpu().numpy()
+    ref = c_oracle.decode(L["packed"], L["tlut"], m, k, K)
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+def test_zero_stream_known_answer(K):
+    # qtip-kernels/src/test.cu:23-58 at a reduced size plus the original 8192^2 for K=2
+    from qtip_amd import ops
+    for m, k in [(64, 256)] + ([(8192, 8192)] if K == 2 else []):
+        pk = torch.zeros(m * k * K // 16, dtype=torch.int16, device="cuda")
+        ones = torch.ones(512, 2, dtype=torch.float16, device="cuda")
+        x = torch.ones(k, dtype=torch.float16, device="cuda")
+        out = ops.decompress_matvec(pk, x, ones, m, k, K)
+        assert torch.all(out == float(k))
+        assert torch.all(ops.decode(pk, ones, m, k, K) == 1.0)
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("shape", SMALL + [(4096, 4096), (4096, 11008), (128, 28672)])
+@pytest.mark.parametrize("split", [True, False])
+def test_matvec_vs_oracle(K, shape, split):
+    from qtip_amd import ops
+    m, k = shape
+    L = make_layer(m, k, K, seed=3 * m + k + K)
+    x = L["x"].reshape(-1)
+    got = ops.decompress_matvec(dev(L["packed"]), dev(x), dev(L["tlut"]), m, k, K, split_k=split).cpu().numpy()
+    ref = c_oracle.matvec(L["packed"], x, L["tlut"], m, k, K)
+    assert_close(got, ref)
+    # the reference's own check (test_decompress_matvec.py:286-294): fp16, atol 1e-5, rtol 1e-2,
+    # on its input scale (codebook and x ~ N(0,1)/16)
+    xs = (L["x"].reshape(-1) / 16).astype(np.float16)
+    ts = (L["tlut"] / 16).astype(np.float16)
+    got2 = ops.decompress_matvec(dev(L["packed"]), dev(xs), dev(ts), m, k, K, split_k=split).cpu().numpy()
+    ref2 = c_oracle.matvec(L["packed"], xs, ts, m, k, K)
+    np.testing.assert_allclose(got2.astype(np.float16).astype(np.float64), ref2.astype(np.float16).astype(np.float64),
+                               atol=1e-5 + 2e-3 * np.abs(ref2).max(), rtol=1e-2)
+
+
+def test_matvec_deterministic_and_workspace_clean():
+    from qtip_amd import ops
+    m, k, K = 4096, 4096, 2
+    L = make_layer(m, k, K, seed=11)
+    pk, x, tl = dev(L["packed"]), dev(L["x"].reshape(-1)), dev(L["tlut"])
+    a = ops.decompress_matvec(pk, x, tl, m, k, K)
+    for _ in range(5):
+        b = ops.decompress_matvec(pk, x, tl, m, k, K)
+        assert torch.equal(a, b)
+
+
+def test_matvec_full_size_properties():
+    # 70B-shaped matrix: linearity in x and agreement with a dense product of
+    # the HIP-decoded weights (decode itself is bit-exact-tested above)
+    from qtip_amd import ops
+    m, k, K = 8192, 28672, 2
+    g = torch.Generator().manual_seed(0)
+    pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+    tl = torch.randn(512, 2, generator=g).half().cuda()
+    x1 = torch.randn(k, generator=g).half().cuda()
+    w = ops.decode(pk, tl, m, k, K)
+    y1 = ops.decompress_matvec(pk, x1, tl, m, k, K)
+    ref = (w.double() @ x1.double()).cpu().numpy()
+    assert_close(y1.cpu().numpy(), ref)
+    y2 = ops.decompress_matvec(pk, (x1 * 2).half(), tl, m, k, K)
+    assert torch.allclose(y2, 2 * y1, rtol=1e-5, atol=1e-3)
+    # checksum of checksums: column sums of the decoded matrix dotted with x
+    np.testing.assert_allclose(float(y1.double().sum()), float((w.double().sum(0) @ x1.double())), rtol=1e-4)
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("shape", [(64, 96), (256, 256), (512, 1024 + 32)])
+@pytest.mark.parametrize("batch", [1, 2, 8, 16, 17, 32, 33, 64, 70])
+def test_gemm_vs_oracle(K, shape, batch):
+    from qtip_amd import ops
+    m, k = shape
+    L = make_layer(m, k, K, seed=m + k + K + batch)
+    rng = np.random.default_rng(batch)
+    X = rng.standard_normal((batch, k)).astype(np.float16)
+    got = ops.decompress_gemm(dev(L["packed"]), dev(X), dev(L["tlut"]), m, k, K, round_f16=False).cpu().numpy()
+    w = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float64)
+    ref = X.astype(np.float64) @ w.T
+    assert_close(got, ref)
+    got16 = ops.decompress_gemm(dev(L["packed"]), dev(X), dev(L["tlut"]), m, k, K, round_f16=True).cpu().numpy()
+    assert np.array_equal(got16, got.astype(np.float16).astype(np.float32))
+
+
+@pytest.mark.parametrize("n", [64, 256, 1024, 4096, 8192, 32768])
+@pytest.mark.parametrize("rows", [1, 3])
+def test_rht_pow2(n, rows):
+    import qtip_amd.utils.matmul_had  # registers hadamard::hadamard
+    from qtip_amd import ops
+    rng = np.random.default_rng(n + rows)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    got = ops.rht(dev(x)).cpu().numpy()
+    ref = O.hadamard_transform(x)
+    assert_close(got, ref, 1e-5, 1e-5)
+    got_op = torch.ops.hadamard.hadamard(dev(x), 0.25).cpu().numpy()
+    assert_close(got_op, ref * np.sqrt(n) * 0.25, 1e-5, 1e-5)
+
+
+@pytest.mark.parametrize("n", [12 * 64, 11008, 22016, 12288, 10240, 28672, 57344, 52 * 256])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_rht_tables(n, transpose):
+    from qtip_amd.utils import matmul_had as mh
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal((2, n)).astype(np.float32)
+    hadK, K = mh.get_hadK(n)
+    fn = mh.matmul_hadUt_cuda if transpose else mh.matmul_hadU_cuda
+    got = fn(dev(x), hadK, K).cpu().numpy()
+    assert_close(got, O.hadamard_transform(x, transpose=transpose), 1e-5, 1e-5)
+    # caller-supplied table tensor (as QuantizedLinear passes it) gives the same
+    got2 = fn(dev(x), hadK.clone().cuda(), K).cpu().numpy()
+    assert np.array_equal(got, got2)
+
+
+def test_rht_fused_sign_scale_and_parts():
+    from qtip_amd import ops
+    from qtip_amd.utils import matmul_had as mh
+    n = 11008
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, 3, n)).astype(np.float32)  # 2 parts, 3 rows
+    pre = np.sign(rng.standard_normal(n)).astype(np.float16)
+    post = rng.standard_normal(n).astype(np.float32)
+    bits = mh.had_bits(None, 172, True, "cuda")
+    got = ops.rht(dev(x), order=172, had_bits=bits, pre=dev(pre), post=dev(post), scale=0.5, out_dtype=torch.float16,
+                  in_parts=2).cpu().numpy()
+    ref = O.hadamard_transform((x[0] + x[1]) * pre.astype(np.float32), transpose=True) * np.sqrt(n) * 0.5 * post
+    assert_close(got, ref, 2e-3, 5e-4)  # fp16 output rounding
+
+
+LAYERS = [(4096, 4096, 2), (4096, 11008, 3), (12288, 4096, 4), (1280, 8192, 2), (256, 28672, 2), (3584, 1024, 2)]
+
+
+@pytest.mark.parametrize("m,n,K", LAYERS)
+@pytest.mark.parametrize("bs", [1, 5])
+def test_bitshift_linear_forward(m, n, K, bs):
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    L = make_layer(m, n, K, seed=m + n + K)
+    rng = np.random.default_rng(bs)
+    inp = rng.standard_normal((bs, n)).astype(np.float16)
+    layer = BitshiftLinear(16, 16, 16, K, 2, 9, 'quantlut_sym', tlut=dev(L["tlut"]), has_kernel=True)
+    had_l, K_l = mh.get_hadK(n)
+    had_r, K_r = mh.get_hadK(m)
+    out = layer(dev(inp), dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), had_l, had_r, K_l, K_r, 0, 8)
+    assert out.dtype == torch.float16 and out.shape == (bs, m)
+    ref = O.bitshift_linear_forward(inp, L["packed"], L["SU"], L["SV"], L["tlut"], K)
+    assert_close(out.cpu().numpy(), ref)
+
+
+def test_bitshift_linear_matches_dense_equivalent():
+    # the reference's own dense form of the layer (bitshift.py:389-413)
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    m, n, K = 12 * 32, 512, 2
+    L = make_layer(m, n, K, seed=2)
+    layer = BitshiftLinear(16, 16, 16, K, 2, 9, 'quantlut_sym', tlut=dev(L["tlut"]), has_kernel=True)
+    had_l, K_l = mh.get_hadK(n)
+    had_r, K_r = mh.get_hadK(m)
+    out = layer(dev(L["x"]), dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), had_l, had_r, K_l, K_r, 0, 8)
+    W = O.dense_equivalent(L["packed"], L["SU"], L["SV"], L["tlut"], K)
+    assert_close(out.cpu().numpy(), L["x"].astype(np.float64) @ W.T)
+
+
+def test_op_names_and_glue():
+    import qtip_amd.codebook as cbk
+    m, k, K = 4096, 4096, 2
+    L = make_layer(m, k, K, seed=9)
+    op = getattr(torch.ops.quip_lib, f"decompress_matvec_qtip_{m}_1_{k}_{K}")
+    out = op(dev(L["packed"]), dev(L["x"]).float(), dev(L["tlut"]))  # fp32 x as the reference passes it
+    assert out.shape == (1, m) and out.dtype == torch.float32
+    ref = c_oracle.matvec(L["packed"], L["x"].reshape(-1), L["tlut"], m, k, K)
+    assert_close(out.cpu().numpy().reshape(-1), ref)
+    assert len(cbk.kernels) >= 61
+
+
+def test_errors_raise_not_exit():
+    from qtip_amd import ops
+    L = make_layer(64, 64, 2)
+    pk, tl, x = dev(L["packed"]), dev(L["tlut"]), dev(L["x"].reshape(-1))
+    with pytest.raises(ValueError):
+        ops.decompress_matvec(pk, x, tl, 64, 96, 2)  # size mismatch
+    with pytest.raises(ValueError):
+        ops.decompress_matvec(pk, x, tl, 64, 64, 5)
+    with pytest.raises(TypeError):
+        ops.decompress_matvec(pk, x.float(), tl, 64, 64, 2)
+    with pytest.raises(ValueError):
+        ops.decompress_matvec(pk.cpu(), x, tl, 64, 64, 2)
+    with pytest.raises(ValueError):
+        ops.decode(pk, tl[:100], 64, 64, 2)
+    with pytest.raises(ValueError):
+        ops.rht(torch.zeros(3, 100, device="cuda"))
+
+
+def test_graph_capture_replays():
+    # the forward path must be capturable (no allocation-free requirement on
+    # torch's side: outputs come from the graph's private pool)
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    m, n, K = 4096, 4096, 2
+    L = make_layer(m, n, K, seed=4)
+    layer = BitshiftLinear(16, 16, 16, K, 2, 9, 'quantlut_sym', tlut=dev(L["tlut"]), has_kernel=True)
+    had_l, K_l = mh.get_hadK(n)
+    had_r, K_r = mh.get_hadK(m)
+    args = (dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), had_l, had_r, K_l, K_r, 0, 8)
+    static_in = dev(L["x"]).clone()
+    eager = layer(static_in, *args).clone()
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            layer(static_in, *args)
+    torch.cuda.current_stream().wait_stream(s)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        static_out = layer(static_in, *args)
+    for it in range(4):
+        xin = dev(L["x"]) * (it + 1)
+        static_in.copy_(xin)
+        g.replay()
+        torch.cuda.synchronize()
+        ref = layer(xin, *args)
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, ref), it
+    assert torch.equal(layer(dev(L["x"]), *args), eager)

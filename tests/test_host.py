@@ -1,0 +1,147 @@
+"""CPU: host logic and the C-ABI surface (no kernel launches)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qtip_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qtip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from qtip_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build with python -m qtip_amd.build"
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared_symbols()
+    assert len(declared) >= 7
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert sorted(_lib.EXPORTED_SYMBOLS) == declared
+    assert _lib.lib().qtip_abi_version() == _lib.ABI_VERSION
+    assert b"shape" in _lib.lib().qtip_error_string(-1)
+
+
+def test_argument_rejection_without_gpu():
+    # rejected arguments return a negative code before anything touches the device
+    from qtip_amd import _lib
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    null = ctypes.c_void_p(0)
+    assert L.qtip_decompress_matvec(p, p, p, p, 33, 64, 2, null, 0, null) == -1
+    assert L.qtip_decompress_matvec(p, p, p, p, 64, 64, 5, null, 0, null) == -1
+    assert L.qtip_decompress_matvec(null, p, p, p, 64, 64, 2, null, 0, null) == -2
+    assert L.qtip_decode(p, p, null, 64, 64, 2, null) == -2
+    assert L.qtip_decompress_gemm(p, p, p, p, 64, 64, 2, 0, 0, null) == -1
+    assert L.qtip_rht(p, 0, p, 0, 1, 1, 100, 1, null, null, null, 1.0, null) == -1  # not a power of two
+    assert L.qtip_rht(p, 0, p, 0, 1, 1, 12 * 64, 12, null, null, null, 1.0, null) == -2  # table missing
+    assert L.qtip_rht(p, 7, p, 0, 1, 1, 64, 1, null, null, null, 1.0, null) == -5
+    assert L.qtip_matvec_workspace_bytes(4096, 4096, 2) >= 16 * 4096 * 4
+
+
+def test_cpu_tensors_raise():
+    from qtip_amd import ops
+    with pytest.raises(ValueError):
+        ops.decode(torch.zeros(64 * 64 * 2 // 16, dtype=torch.int16), torch.zeros(512, 2, dtype=torch.float16), 64, 64, 2)
+    import qtip_amd.utils.matmul_had  # registers hadamard::hadamard (GPU implementation only)
+    with pytest.raises(NotImplementedError):
+        torch.ops.hadamard.hadamard(torch.zeros(2, 64), 1.0)
+
+
+def test_has_kernel_gate():
+    from qtip_amd.utils.kernel_check import has_kernel
+    assert has_kernel('quantlut_sym', 16, 2, 2, 9, 16, 16)
+    assert has_kernel('quantlut_sym', 16, 4, 2, 9, 16, 16)
+    for bad in [('lut', 16, 2, 2, 9, 16, 16), ('quantlut_sym', 12, 2, 2, 9, 16, 16), ('quantlut_sym', 16, 5, 2, 9, 16, 16),
+                ('quantlut_sym', 16, 1, 2, 9, 16, 16), ('quantlut_sym', 16, 2, 1, 9, 16, 16),
+                ('quantlut_sym', 16, 2, 2, 10, 16, 16), ('quantlut_sym', 16, 2, 2, 9, 8, 16)]:
+        assert not has_kernel(*bad)
+
+
+def test_op_registry_names():
+    import qtip_amd.codebook as cbk
+    # every BASELINE shape at every bit width, under the reference's naming scheme
+    for m, k in [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (10240, 8192), (8192, 8192),
+                 (57344, 8192), (8192, 28672), (28672, 8192)]:
+        for b in (2, 3, 4):
+            assert (m, 1, k, b) in cbk.kdict
+            assert hasattr(torch.ops.quip_lib, f"decompress_matvec_qtip_{m}_1_{k}_{b}")
+    assert len([k for k in cbk.kernels if k[0] != 256]) == 61
+    op = cbk.register_shape(64, 128, 3)
+    assert op is cbk.kdict[(64, 1, 128, 3)]
+    with pytest.raises(ValueError):
+        cbk.register_shape(48, 128, 3)
+    # fake (meta) implementation: shape/dtype only
+    out = torch.ops.quip_lib.decompress_matvec_qtip_4096_1_4096_2(
+        torch.empty(1, device="meta", dtype=torch.int16), torch.empty(1, 4096, device="meta"),
+        torch.empty(512, 2, device="meta", dtype=torch.float16))
+    assert out.shape == (1, 4096) and out.dtype == torch.float32
+
+
+def test_quantlut_sym_matches_oracle():
+    from oracle import qtip_oracle as O
+    from qtip_amd.codebook.bitshift import quantlut_sym
+    t = torch.randn(512, 2, generator=torch.Generator().manual_seed(0)).half()
+    a = quantlut_sym(t, 16, 9).numpy().view(np.uint16)
+    b = O.quantlut_sym(t.numpy()).view(np.uint16)
+    assert np.array_equal(a, b)
+
+
+def test_tlut_roundtrip_through_expanded_table():
+    from qtip_amd.codebook.bitshift import quantlut_sym
+    from qtip_amd.utils.kernel_decompress import _representatives, tlut_from_expanded
+    t = torch.randn(512, 2, generator=torch.Generator().manual_seed(1)).half()
+    back = tlut_from_expanded(quantlut_sym(t, 16, 9))
+    seen = _representatives()[2]
+    assert torch.equal(back[seen], t[seen])
+    # every index some state hashes to is covered (all 512 are reachable)
+    assert int(seen.sum()) == 512
+
+
+def test_unpack_trellis_matches_oracle():
+    from oracle import qtip_oracle as O
+    from qtip_amd.codebook.bitshift import bitshift_codebook
+    for K in (2, 3, 4):
+        cb = bitshift_codebook(16, K, 2, 9, 'quantlut_sym', tlut=torch.zeros(512, 2, dtype=torch.float16))
+        words = np.random.default_rng(K).integers(0, 65536, (6, 16 * K), dtype=np.uint16)
+        got = cb.unpack_trellis(torch.from_numpy(words.view(np.int16)), 256).numpy()
+        assert np.array_equal(got, O.unpack_trellis_natural(words, K))
+
+
+def test_get_hadK_and_bits():
+    from oracle import qtip_oracle as O
+    from qtip_amd.utils import matmul_had as mh
+    for n in (4096, 11008, 12288, 10240, 28672, 57344, 22016):
+        had, K = mh.get_hadK(n)
+        ohad, oK = O.get_hadK(n)
+        assert K == oK
+        if K > 1:
+            assert np.array_equal(had.numpy(), ohad)
+            assert np.array_equal(mh.get_hadK(n, transpose=True)[0].numpy(), ohad.T)
+    with pytest.raises(AssertionError):
+        mh.get_hadK(100)
+    neg = np.random.default_rng(0).integers(0, 2, (20, 20)).astype(bool)
+    w = mh._pack_bits(neg).view(np.uint32)
+    for i in range(20):
+        for j in range(20):
+            b = i * 20 + j
+            assert ((w[b >> 5] >> (b & 31)) & 1) == neg[i, j]
+
+
+def test_quantiser_entry_points_raise():
+    from qtip_amd.codebook.bitshift import BitshiftLinear, bitshift_codebook
+    cb = bitshift_codebook(16, 2, 2, 9, 'quantlut_sym')
+    with pytest.raises(NotImplementedError):
+        cb.quantize(None)
+    with pytest.raises(NotImplementedError):
+        bitshift_codebook(16, 2, 1, 16, '1mad')
+    with pytest.raises(ValueError):
+        BitshiftLinear(16, 16, 16, 5, 2, 9, 'quantlut_sym', has_kernel=True)
