@@ -53,10 +53,15 @@ const char* qtip_error_string(int code);
 int qtip_decode(void* out_f16, const void* packed, const void* tlut,
                 int m, int k, int bits, void* stream);
 
-/* Bytes of scratch qtip_decompress_matvec wants for this shape (0 = none).
- * Its first 64 KiB (arrival counters) must be zero before the first use; every
- * call leaves them zero again, so one buffer can serve calls of any shape.
- * Calls that share one scratch buffer must not overlap in time. */
+/* Number of k splits S (>= 1) the matvec uses for this shape on the current
+ * device: small m cannot fill 256 CUs with 32-row blocks alone, so the k
+ * dimension is cut into S ranges whose partial sums are added afterwards in a
+ * fixed order.  Returns 0 for an unsupported shape. */
+int qtip_matvec_split(int m, int k, int bits);
+
+/* Bytes of scratch qtip_decompress_matvec wants for this shape: S*m floats
+ * when S > 1, else 0.  The scratch needs no initialisation.  Calls that share
+ * one scratch buffer must not overlap in time. */
 size_t qtip_matvec_workspace_bytes(int m, int k, int bits);
 
 /* bs=1 decompress + matvec: out[m] (fp32) = hatW[m][k] . x[k] (fp16), fp32
@@ -66,11 +71,20 @@ size_t qtip_matvec_workspace_bytes(int m, int k, int bits);
  * inference.cu:432-471) and the 64 pybind entry points
  * decompress_matvec_16_9_{R}_1_{M}_1_{K} (qtip-kernels/src/wrapper.cpp:489-564).
  * Shapes are run-time arguments: m % 32 == 0, k % 32 == 0, bits in {2,3,4}.
- * `workspace` may be NULL (then the k dimension is never split across
- * workgroups, which costs parallelism on small m). */
+ * With a workspace and S > 1 this is two launches (partial sums, then their
+ * sum); `workspace` may be NULL, then k is never split (one launch, less
+ * parallelism on small m). */
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16,
                            const void* tlut, int m, int k, int bits,
                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same kernel, but leaves the nparts partial vectors parts[nparts][m] for the
+ * consumer to add (qtip_rht does so on load through its in_parts argument),
+ * which saves the second launch inside BitshiftLinear.forward.
+ * 1 <= nparts <= 16; normally nparts = qtip_matvec_split(m, k, bits). */
+int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x_f16,
+                                 const void* tlut, int m, int k, int bits, int nparts,
+                                 void* stream);
 
 /* Batched decompress + GEMM on the matrix cores:
  * out[batch][m] = x[batch][k] (fp16) . hatW[m][k]^T, fp32 accumulate.

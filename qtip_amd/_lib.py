@@ -9,11 +9,11 @@ import os
 import torch  # must be imported first so that its bundled HIP runtime is the one libqtip_hip.so binds to
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libqtip_hip.so")
+LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hip.so")
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 
@@ -26,7 +26,9 @@ _SIGNATURES = {
     "qtip_abi_version": (ctypes.c_int, []),
     "qtip_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "qtip_decode": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p]),
+    "qtip_matvec_split": (ctypes.c_int, [ctypes.c_int] * 3),
     "qtip_matvec_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
+    "qtip_decompress_matvec_parts": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "qtip_decompress_matvec": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
                                [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "qtip_decompress_gemm": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_void_p]),

@@ -14,7 +14,6 @@ from torch import nn
 from .. import ops
 from ..utils.kernel_check import has_kernel as _has_kernel
 from ..utils.matmul_had import had_bits, matmul_hadU_cuda, matmul_hadUt_cuda
-from . import kdict, register_shape
 
 
 def quantlut_sym(tlut, L, nbits):
@@ -172,12 +171,14 @@ class BitshiftLinear(nn.Module):
                          scale=(nn_**-0.5) / self.scale, out_dtype=torch.float16).reshape(bs, n)
 
         # ---- quantised matmul
+        in_parts = 1
         if self.has_kernel:
             tl = self._tlut16(dev)
             if bs == 1:
-                key = (m, 1, n, self.cb.K)
-                wrapper = kdict.get(key) or register_shape(m, n, self.cb.K)
-                y = wrapper(trellis, xt, tl)
+                # same kernel as the quip_lib::decompress_matvec_qtip_* op; the k-split
+                # partial sums (if any) are added by the output transform on load
+                y = ops.decompress_matvec_parts(trellis.reshape(-1), xt.reshape(-1), tl.reshape(-1), m, n, self.cb.K)
+                in_parts = y.shape[0]
             else:
                 y = ops.decompress_gemm(trellis.reshape(-1), xt, tl, m, n, self.cb.K, round_f16=True)
         else:
@@ -189,10 +190,13 @@ class BitshiftLinear(nn.Module):
         fused_out = (rcp != 2 and SV.dtype == torch.float32 and SV.device == dev
                      and input.dtype in (torch.float16, torch.float32))
         if fused_out:
-            out = ops.rht(y, order=K_right,
+            out = ops.rht(y if in_parts > 1 else y.reshape(bs, m), order=K_right,
                           had_bits=had_bits(had_right, K_right, False, dev) if K_right > 1 else None,
-                          post=SV.contiguous(), scale=(m**-0.5) * self.scale, out_dtype=input.dtype)
+                          post=SV.contiguous(), scale=(m**-0.5) * self.scale, out_dtype=input.dtype,
+                          in_parts=in_parts)
         else:
+            if in_parts > 1:
+                y = y.sum(0, keepdim=True)
             yy = y.reshape(-1, m // tp_rank) if rcp == 2 else y
             mm = yy.shape[-1]
             yt = ops.rht(yy.contiguous(), order=K_right,

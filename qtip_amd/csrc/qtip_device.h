@@ -172,4 +172,171 @@ __device__ __forceinline__ uint32_t lut_lookup(const uint32_t* lut, uint32_t s, 
   return *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(lut) + addr);
 }
 
+// ---------------------------------------------------------------------------
+// Fast path of the matvec: conflict-free table and packed 16-bit hashing.
+//
+// Table: 1024 entries x 32 replicas x 4 bytes = 128 KiB, entry e at byte
+// e*128, replica (lane % 32) at +4*(lane%32): every lane of a half-wave reads
+// its own LDS bank, so a gather of 64 random entries takes the same time as a
+// broadcast.  Two states travel in one register (16 bits each):
+//   hash      v_pk_mad_u16  p = s*s + s           (one instruction, two states)
+//   mask      v_and_b32     q = p & 0xFFC0FFC0    (bits 6..15 = entry, both halves)
+//   address   v_mad_u32_u16 a = q.half * 2 + slot4 (op_sel picks the half)
+// The instructions are written as inline asm because the compiler rewrites
+// s*s+s into add+mul and picks 64-bit multiplies for the unpacked form.
+// ---------------------------------------------------------------------------
+constexpr int kLut128Bytes = kLutEntries * 128;
+
+__device__ __forceinline__ void build_lut128(uint32_t* lut, const uint32_t* __restrict__ tlut,
+                                             int tid, int nthreads) {
+  // thread handles (entry, quarter): 32 bytes x 4 quarters... one u32x4 per step
+  for (int i = tid; i < kLutEntries * 8; i += nthreads) {
+    const int e = i >> 3;
+    uint32_t w = tlut[e & 511] ^ ((uint32_t)(e >> 9) << 15);
+    u32x4 v = {w, w, w, w};
+    reinterpret_cast<u32x4*>(lut)[i] = v;
+  }
+}
+
+// p.lo = s.lo*s.lo + s.lo, p.hi = s.hi*s.hi + s.hi (mod 2^16 each)
+__device__ __forceinline__ uint32_t pk_hash(uint32_t s) {
+  uint32_t r;
+  asm("v_pk_mad_u16 %0, %1, %1, %1" : "=v"(r) : "v"(s));
+  return r;
+}
+// per half: a * c + b (mod 2^16); cst holds the same 16-bit constant in both halves
+__device__ __forceinline__ uint32_t pk_mad_const(uint32_t a, uint32_t cst, uint32_t b) {
+  uint32_t r;
+  asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(cst), "v"(b));
+  return r;
+}
+__device__ __forceinline__ uint32_t pk_shr(uint32_t a, int sh) {
+  typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+  u16x2 v = __builtin_bit_cast(u16x2, a);
+  v = v >> (u16x2)(uint16_t)sh;
+  return __builtin_bit_cast(uint32_t, v);
+}
+// unpacked hash (only the low 16 bits of s and of the result are meaningful)
+__device__ __forceinline__ uint32_t hash24(uint32_t s) {
+  uint32_t r;
+  asm("v_mad_u32_u24 %0, %1, %1, %1" : "=v"(r) : "v"(s));
+  return r;
+}
+// LDS byte address of the entry selected by the low / high half of q = p & 0xFFC0FFC0
+__device__ __forceinline__ uint32_t lut128_addr_lo(uint32_t q, uint32_t slot4) {
+  uint32_t r;
+  asm("v_mad_u32_u16 %0, %1, 2, %2 op_sel:[0,0,0,0]" : "=v"(r) : "v"(q), "v"(slot4));
+  return r;
+}
+__device__ __forceinline__ uint32_t lut128_addr_hi(uint32_t q, uint32_t slot4) {
+  uint32_t r;
+  asm("v_mad_u32_u16 %0, %1, 2, %2 op_sel:[1,0,0,0]" : "=v"(r) : "v"(q), "v"(slot4));
+  return r;
+}
+// ---------------------------------------------------------------------------
+// Packed state extraction: 16 registers per lane per wave-load, two 16-bit
+// states in each.  Register i and half h (0 = low) stand for
+//   K = 2,3:  i = (R*2 + kh)*4 + j,  half h -> tile row half mh = h
+//   K = 4:    i = (R*4 + 2*kh + mh)*2 + u,  half h -> j = 2*(1-h) + u
+// (R = ref lane A/B, j = state inside the chunk = 2*jh + rh).  pk_meta gives
+// the x pair (2*kh + jh) and the accumulator (2*mh + rh) of a half.
+// ---------------------------------------------------------------------------
+template <int K>
+struct PkMeta {
+  static constexpr __device__ int R(int i) { return K == 4 ? (i >> 3) : (i >> 3); }
+  static constexpr __device__ int xq(int i, int h) {
+    if (K == 4) {
+      const int kh = (i >> 2) & 1, u = i & 1, j = 2 * (1 - h) + u;
+      return 2 * kh + (j >> 1);
+    }
+    const int kh = (i >> 2) & 1, j = i & 3;
+    return 2 * kh + (j >> 1);
+  }
+  static constexpr __device__ int acc(int i, int h) {
+    if (K == 4) {
+      const int mh = (i >> 1) & 1, u = i & 1, j = 2 * (1 - h) + u;
+      return 2 * mh + (j & 1);
+    }
+    const int j = i & 3;
+    return 2 * h + (j & 1);
+  }
+};
+
+__device__ __forceinline__ uint32_t perm(uint32_t hi_src, uint32_t lo_src, uint32_t sel) {
+  // result byte b = selector byte b: 0..3 -> lo_src byte, 4..7 -> hi_src byte
+  return __builtin_amdgcn_perm(hi_src, lo_src, sel);
+}
+
+template <int K>
+__device__ __forceinline__ void packed_states(const LaneData<K>& ld, uint32_t P[16]) {
+  if constexpr (K == 2) {
+    // dword R*2+kh = chunk(mh=0) | chunk(mh=1) << 16; a chunk is 4 states of 4 bits
+    const uint32_t nb0 = from_next_lane16(ld.d[0]);
+    const uint32_t nb1 = from_next_lane16(ld.d[1]);
+#pragma unroll
+    for (int R = 0; R < 2; ++R)
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) {
+        const uint32_t d = ld.d[R * 2 + kh];
+        const uint32_t n = R == 0 ? ld.d[2 + kh] : (kh == 0 ? nb0 : nb1);
+        uint32_t* o = &P[(R * 2 + kh) * 4];
+        o[0] = d;
+        o[1] = pk_mad_const(d, 0x00100010u, pk_shr(n, 12));  // d<<4 | n>>12
+        o[2] = perm(d, n, 0x06030401u);                       // d<<8 | n>>8
+        o[3] = pk_mad_const(d, 0x10001000u, pk_shr(n, 4));   // d<<12 | n>>4
+      }
+  } else if constexpr (K == 3) {
+    // 24-bit chunks c at byte 3t of the ref lane's 12 bytes.  Per tile pair:
+    // X1 = c[23:8] (= state 0), X2 = c[15:0], NX = X1 of the successor.
+    uint32_t X1[2][2], X2[2][2];
+#pragma unroll
+    for (int R = 0; R < 2; ++R) {
+      const uint32_t e0 = ld.d[3 * R], e1 = ld.d[3 * R + 1], e2 = ld.d[3 * R + 2];
+      X1[R][0] = perm(e0, e1, 0x01000605u);
+      X2[R][0] = perm(e0, e1, 0x00070504u);
+      X1[R][1] = perm(e1, e2, 0x03020007u);
+      X2[R][1] = perm(e1, e2, 0x02010706u);
+    }
+    const uint32_t nb0 = from_next_lane16(X1[0][0]);
+    const uint32_t nb1 = from_next_lane16(X1[0][1]);
+#pragma unroll
+    for (int R = 0; R < 2; ++R)
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) {
+        const uint32_t x1 = X1[R][kh], x2 = X2[R][kh];
+        const uint32_t nx = R == 0 ? X1[1][kh] : (kh == 0 ? nb0 : nb1);
+        uint32_t* o = &P[(R * 2 + kh) * 4];
+        o[0] = x1;                                                      // c[23:8]
+        o[1] = pk_mad_const(pk_shr(x1, 8), 0x40004000u, pk_shr(x2, 2));  // c[17:2]
+        o[2] = pk_mad_const(x2, 0x00100010u, pk_shr(nx, 12));           // c[11:0] | nx[15:12]
+        o[3] = pk_mad_const(x2, 0x04000400u, pk_shr(nx, 6));            // c[5:0] | nx[15:6]
+      }
+  } else {
+    // 32-bit chunk c: states c[31:16], c[23:8], c[15:0], c[7:0] | next[31:24]
+    uint32_t nb[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) nb[t] = from_next_lane16(ld.d[t]);
+#pragma unroll
+    for (int R = 0; R < 2; ++R)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t c = ld.d[R * 4 + t];
+        const uint32_t cn = R == 0 ? ld.d[4 + t] : nb[t];
+        P[(R * 4 + t) * 2] = c;                             // hi = state 0, lo = state 2
+        P[(R * 4 + t) * 2 + 1] = perm(c, cn, 0x06050403u);  // hi = state 1, lo = state 3
+      }
+  }
+}
+
+// 32-bit LDS address of a __shared__ object and a load from such an address:
+// with the table base folded into the per-lane slot offset, the address that
+// v_mad_u32_u16 produces feeds ds_read_b32 directly (no per-lookup add).
+typedef __attribute__((address_space(3))) const uint32_t lds_u32_t;
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+__device__ __forceinline__ uint32_t lds_word_abs(uint32_t lds_addr) {
+  return *(lds_u32_t*)(uintptr_t)lds_addr;
+}
+
 }  // namespace qtip

@@ -14,7 +14,6 @@ namespace {
 constexpr int kThreads = 1024;  // 16 waves per workgroup, one workgroup per CU
 constexpr int kWaves = kThreads / 64;
 constexpr int kMaxSplit = 16;
-constexpr size_t kCounterBytes = 65536;  // arrival counters at the start of the matvec workspace
 
 __device__ __forceinline__ float dpp_xor1(float v) {
   return __builtin_bit_cast(
@@ -81,134 +80,225 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // ---------------------------------------------------------------------------
 // decompress + matvec
 // ---------------------------------------------------------------------------
+constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
+
+// 32 states of one wave-load.  All hashes, addresses and the 32 table reads
+// are issued first and the 32 dot products follow, so a read has the rest of
+// the address arithmetic (a few hundred cycles) to come back from LDS.
+// slot4 = LDS address of the table + 4 * (lane % 32);
+// acc[2*mh + rh] belongs to row 16*mh + 8*rh + a/2 of the 32-row block.
 template <int K>
-__device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld,
-                                                  const uint16_t* __restrict__ xp,
-                                                  const uint32_t* lut, uint32_t slot4,
-                                                  float acc[4]) {
-  // x for columns 8*q + 4*(a%2) + {0..3}, q = 2*kh + jh
-  u32x2 xv[4];
+__device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u32x2 xv[4],
+                                                  uint32_t slot4, float acc[4]) {
+  uint32_t P[16], W[32];
+  packed_states<K>(ld, P);
 #pragma unroll
-  for (int q = 0; q < 4; ++q) xv[q] = *reinterpret_cast<const u32x2*>(xp + 8 * q);
-  uint32_t st[2][4][4];
-  lane_states<K>(ld, st);
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
+#if defined(QTIP_ABLATE_LDS)
+    W[2 * i] = lut128_addr_lo(q, slot4);
+    W[2 * i + 1] = lut128_addr_hi(q, slot4);
+#else
+    W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
+    W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
+#endif
+  }
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int kh = t >> 1, mh = t & 1;
+  for (int i = 0; i < 16; ++i) {
+    const int R = PkMeta<K>::R(i);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int jh = j >> 1, rh = j & 1;
+    for (int hh = 0; hh < 2; ++hh) {
+      // (copy the vector element to a scalar first: bit_cast applied directly
+      // to a vector-element lvalue reads element 0)
+      const uint32_t xr = xv[PkMeta<K>::xq(i, hh)][R];
+      acc[PkMeta<K>::acc(i, hh)] =
+          __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, W[2 * i + hh]),
+                                 __builtin_bit_cast(half2_t, xr), acc[PkMeta<K>::acc(i, hh)], false);
+    }
+  }
+}
+
+// Buffer-addressed streaming loads: the address is (SGPR descriptor, SGPR byte
+// offset, per-lane VGPR offset), so walking the stream costs no vector ALU work.
+template <int K>
+__device__ __forceinline__ LaneData<K> load_lane_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
+                                                     uint32_t soff) {
+  LaneData<K> r;
+  constexpr int NT = 2;  // non-temporal: the stream is read once
+  if constexpr (K == 2) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
 #pragma unroll
-      for (int R = 0; R < 2; ++R) {
-        const uint32_t w = lut_lookup(lut, st[R][t][j], slot4);
-        // (copy the vector element to a scalar first: bit_cast applied directly
-        // to a vector-element lvalue reads element 0)
-        const uint32_t xr = xv[2 * kh + jh][R];
-        acc[2 * mh + rh] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w),
-                                                  __builtin_bit_cast(half2_t, xr),
-                                                  acc[2 * mh + rh], false);
+    for (int i = 0; i < 4; ++i) r.d[i] = v[i];
+  } else if constexpr (K == 3) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
+    const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff + 16, soff, NT);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.d[i] = v[i];
+    r.d[4] = w[0];
+    r.d[5] = w[1];
+  } else {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
+    const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff + 16, soff, NT);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      r.d[i] = v[i];
+      r.d[4 + i] = w[i];
+    }
+  }
+  return r;
+}
+
+// x for a lane's columns of a wave-load: 4 x (4 consecutive fp16), 16 bytes apart
+__device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff,
+                                           u32x2 xv[4]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) xv[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff + 16 * q, soff, 0);
+}
+
+__device__ __forceinline__ void load_x(const uint16_t* __restrict__ xw, uint32_t xoff, u32x2 xv[4]) {
+  const uint8_t* p = reinterpret_cast<const uint8_t*>(xw) + xoff;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) xv[q] = *reinterpret_cast<const u32x2*>(p + 16 * q);
+}
+
+// Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup take
+// the unit's wave-loads round-robin (so the workgroup streams one contiguous
+// run of bytes), reduce across lanes with DPP / ds_swizzle / permlane swaps and
+// across waves through LDS in a fixed order, and store 32 sums to
+// dst[s*m + 32*rb ...]: the result itself when S == 1, else one of S partial
+// vectors that the consumer adds in order (deterministic either way).
+//
+// The launcher makes gridDim.x a multiple of S: a workgroup keeps one k range
+// [wl0, wl1) and walks row blocks rb0, rb0 + rb_step, ...  A wave sees its work
+// as a flat sequence of items (unit i, j) with wave-load wl0 + wave + 16*j;
+// every unit has npw items per wave of which the first nvj are real (the same
+// count in every unit).  DEPTH items are in flight; the prefetch runs ahead
+// across unit boundaries and every load in the loop is unconditional (a
+// conditional prefetch makes the compiler wait for it at once): padding items
+// fetch offset 0 and are skipped by the arithmetic.
+template <int K, int DEPTH>
+__global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
+    float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut, int m, int k, int S, int wl_per) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+  float* part = reinterpret_cast<float*>(smem + kLut128Bytes);  // [2][kWaves][32]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  const int a = lane & 15, g = lane >> 4;
+  const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
+  const int nkb = k >> 5;
+  const int nwl = (nkb + 3) >> 2;  // wave-loads per row block, the last may be partial
+  const int nfull = nkb >> 2;      // full wave-loads per row block
+  const int nrb = m >> 5;
+  const uint32_t rb_bytes = (uint32_t)nkb * 128 * K;
+  constexpr uint32_t WL_BYTES = 512 * K;
+  const uint32_t loff = (uint32_t)lane * 8 * K;                // lane's bytes inside a wave-load
+  const uint32_t xoff = (uint32_t)(32 * g + 4 * (a & 1)) * 2;  // lane's x bytes inside a wave-load
+
+  const int s = blockIdx.x % S;
+  const int rb0 = blockIdx.x / S;
+  const int rb_step = gridDim.x / S;
+  const int wl0 = s * wl_per;
+  const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
+  const int wl1f = wl1 < nfull ? wl1 : nfull;           // end of the full wave-loads
+  const int npw = (wl_per + kWaves - 1) / kWaves;       // items per wave and unit (padded)
+  const int upw = (nrb - rb0 + rb_step - 1) / rb_step;  // units of this workgroup
+  const int T = upw * npw;
+  const int w_first = wl0 + wave;
+  const int nvj = w_first < wl1f ? (wl1f - w_first + kWaves - 1) / kWaves : 0;  // real items per unit
+  const bool tail_wave = wl1 > nfull && ((nfull - wl0) % kWaves) == wave;
+  float* out_s = dst + (size_t)s * m;
+
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_x =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(x), 0, k * 2, 0x00020000);
+
+  // load cursor: unit l_i (row block l_rb), item l_j
+  int l_j = 0, l_t = 0;
+  uint32_t l_rboff = (uint32_t)rb0 * rb_bytes;
+  const uint32_t rb_step_bytes = (uint32_t)rb_step * rb_bytes;
+  LaneData<K> buf[DEPTH];
+  u32x2 xbuf[DEPTH][4];
+  auto issue = [&](int d) {
+    const bool valid = l_j < nvj && l_t < T;
+    const uint32_t wl = (uint32_t)(w_first + l_j * kWaves);
+    const uint32_t woff = valid ? l_rboff + wl * WL_BYTES : 0u;
+    const uint32_t xw = valid ? wl * 256u : 0u;
+    buf[d] = load_lane_buf<K>(rs_w, loff, woff);
+    load_x_buf(rs_x, xoff, xw, xbuf[d]);
+    ++l_t;
+    if (++l_j == npw) {
+      l_j = 0;
+      l_rboff += rb_step_bytes;
+    }
+  };
+  // the first loads go out before the table is built
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue(d);
+
+  build_lut128(lut, tlut, tid, kThreads);
+  __syncthreads();
+
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  int parity = 0, c_j = 0, c_rb = rb0;
+  for (int t = 0; t < T; t += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (t + d < T) {
+        if (c_j < nvj) matvec_accumulate<K>(buf[d], xbuf[d], slot4, acc);
+      }
+      // the stage's registers are refilled only after their last use, so the
+      // refill reuses them in place (no copies, no wait on the new load)
+      issue(d);
+      if (t + d < T && ++c_j == npw) {
+        // ---- end of a unit: ragged tail, reductions, store
+        // k/32 not a multiple of 4: one wave takes the partial wave-load with
+        // the lanes of the missing blocks switched off
+        if (tail_wave && 4 * nfull + g < nkb) {
+          u32x2 xt[4];
+          load_x(x + (size_t)nfull * 128, xoff, xt);
+          const LaneData<K> tail =
+              load_lane<K>(packed + (size_t)c_rb * rb_bytes + (size_t)nfull * WL_BYTES + loff);
+          matvec_accumulate<K>(tail, xt, slot4, acc);
+        }
+        float* pp = part + parity * (kWaves * 32);
+        // lanes sharing a row differ in lane bits 0 (column half), 4 and 5 (block)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = acc[i];
+          v += dpp_xor1(v);
+          v += swz_xor16(v);
+          v += xor32(v);
+          if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
+          acc[i] = 0.f;
+        }
+        __syncthreads();
+        if (tid < 32) {
+          float sum = 0.f;
+#pragma unroll
+          for (int w = 0; w < kWaves; ++w) sum += pp[w * 32 + tid];
+          out_s[c_rb * 32 + tid] = sum;
+        }
+        parity ^= 1;  // the other buffer is free: its readers passed the barrier above
+        c_j = 0;
+        c_rb += rb_step;
       }
     }
   }
 }
 
-// Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup share
-// a unit's wave-loads round-robin, reduce through LDS in a fixed order and
-// either store the 32 results (S == 1) or publish a partial row block; the
-// last workgroup to arrive for a row block adds the S partials in order
-// 0..S-1, so the result does not depend on scheduling.
-template <int K, int DEPTH>
-__global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
-    float* __restrict__ out, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int S, float* ws, unsigned* counters) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-  float* part = reinterpret_cast<float*>(smem + kLutBytes);  // [kWaves][32]
-  __shared__ int s_last;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int a = lane & 15, g = lane >> 4;
-  const uint32_t slot4 = (uint32_t)a << 2;
-  const int nkb = k >> 5;
-  const int nwl = (nkb + 3) >> 2;
-  const size_t rb_bytes = (size_t)nkb * 128 * K;
-  const int units = (m >> 5) * S;
-  const uint16_t* xlane = x + 4 * (a & 1) + 32 * g;
-  constexpr int WL_BYTES = 512 * K;
-
-  build_lut(lut, tlut, tid, kThreads);
-  __syncthreads();
-
-  for (int u = blockIdx.x; u < units; u += gridDim.x) {
-    const int rb = u / S, s = u - rb * S;
-    const int wl0 = (int)((long)s * nwl / S), wl1 = (int)((long)(s + 1) * nwl / S);
-    const uint8_t* base = packed + (size_t)rb * rb_bytes + (size_t)g * 128 * K + a * 8 * K;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-
-    LaneData<K> buf[DEPTH];
-    int wl = wl0 + wave;
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int w = wl + d * kWaves;
-      if (w < wl1 && 4 * w + g < nkb) buf[d] = load_lane<K>(base + (size_t)w * WL_BYTES);
-    }
-    for (; wl < wl1; wl += DEPTH * kWaves) {
-#pragma unroll
-      for (int d = 0; d < DEPTH; ++d) {
-        const int w = wl + d * kWaves;
-        if (w < wl1) {
-          const LaneData<K> cur = buf[d];
-          const int wn = w + DEPTH * kWaves;
-          if (wn < wl1 && 4 * wn + g < nkb) buf[d] = load_lane<K>(base + (size_t)wn * WL_BYTES);
-          if (4 * w + g < nkb) matvec_accumulate<K>(cur, xlane + (size_t)w * 128, lut, slot4, acc);
-        }
-      }
-    }
-
-    // lanes sharing a row differ in lane bits 0 (column half), 4 and 5 (block)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float v = acc[i];
-      v += dpp_xor1(v);
-      v += swz_xor16(v);
-      v += xor32(v);
-      if (g == 0 && (a & 1) == 0) part[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
-    }
-    __syncthreads();
-    if (tid < 32) {
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) sum += part[w * 32 + tid];
-      if (S == 1) {
-        out[rb * 32 + tid] = sum;
-      } else {
-        __hip_atomic_store(ws + (size_t)s * m + rb * 32 + tid, sum, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    if (S > 1) {
-      __threadfence();
-      __syncthreads();
-      if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(counters + rb, 1u, __ATOMIC_ACQ_REL,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == (unsigned)(S - 1));
-      }
-      __syncthreads();
-      if (s_last) {
-        __threadfence();
-        if (tid < 32) {
-          float sum = 0.f;
-          for (int s2 = 0; s2 < S; ++s2)
-            sum += __hip_atomic_load(ws + (size_t)s2 * m + rb * 32 + tid, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
-          out[rb * 32 + tid] = sum;
-        }
-        if (tid == 0)
-          __hip_atomic_store(counters + rb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    __syncthreads();
-  }
+// out[i] = parts[0][i] + parts[1][i] + ... in that order
+__global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ out,
+                                                        const float* __restrict__ parts, int m,
+                                                        int S) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= m) return;
+  float sum = parts[i];
+  for (int s = 1; s < S; ++s) sum += parts[(size_t)s * m + i];
+  out[i] = sum;
 }
 
 // ---------------------------------------------------------------------------
@@ -443,7 +533,6 @@ hipError_t allow_lds(F* fn, size_t bytes) {
                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-constexpr size_t kMatvecLds = kLutBytes + kWaves * 32 * sizeof(float);
 constexpr size_t kGemmLds = kLutBytes + kGemmWaves * kStageBytes;
 
 hipError_t setup_once() {
@@ -479,7 +568,7 @@ int check_common(const void* a, const void* b, const void* c, const void* d, int
   if (!a || !b || !c || !d) return QTIP_E_NULL;
   if (bits < 2 || bits > 4) return QTIP_E_SHAPE;
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31)) return QTIP_E_SHAPE;
-  if ((long)m * k > (1L << 40)) return QTIP_E_SHAPE;
+  if ((long)m * k * bits / 8 >= (1L << 31)) return QTIP_E_SHAPE;  // 32-bit buffer offsets
   return QTIP_OK;
 }
 
@@ -508,7 +597,7 @@ int choose_split(int m, int k, int bits, int cus) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 1; }
+int qtip_abi_version(void) { return 2; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -547,49 +636,74 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
   return (int)hipGetLastError();
 }
 
-size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
-  (void)k;
-  (void)bits;
-  if (m <= 0) return 0;
-  // fixed-size block of arrival counters (one per 32-row block; the only part
-  // that must stay zero between calls) followed by kMaxSplit partial vectors
-  return kCounterBytes + (size_t)kMaxSplit * m * sizeof(float);
+int qtip_matvec_split(int m, int k, int bits) {
+  if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return 0;
+  return choose_split(m, k, bits, di.cus);
 }
 
-int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,
-                           int m, int k, int bits, void* workspace, size_t workspace_bytes,
-                           void* stream) {
+size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
+  const int S = qtip_matvec_split(m, k, bits);
+  return S > 1 ? (size_t)S * m * sizeof(float) : 0;
+}
+
+static int launch_matvec(float* dst, const void* packed, const void* x_f16, const void* tlut, int m,
+                         int k, int bits, int S, hipStream_t st) {
+  DeviceInfo& di = device_info();
+  const long units = (long)(m >> 5) * S;
+  long grid = units < di.cus ? units : di.cus;
+  grid -= grid % S;  // a workgroup keeps one k range (units is a multiple of S, so grid >= S)
+  const int nwl = ((k >> 5) + 3) >> 2;
+  const int wl_per = (nwl + S - 1) / S;
+  auto* p = (const uint8_t*)packed;
+  auto* xx = (const uint16_t*)x_f16;
+  auto* t = (const uint32_t*)tlut;
+  switch (bits) {
+    case 2: matvec_kernel<2, 4><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+    case 3: matvec_kernel<3, 3><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+    default: matvec_kernel<4, 2><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+  }
+  return (int)hipGetLastError();
+}
+
+static int check_matvec(const void* out, const void* packed, const void* x_f16, const void* tlut,
+                        int m, int k, int bits) {
   int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (!aligned16(packed) || (reinterpret_cast<uintptr_t>(x_f16) & 7u) ||
       (reinterpret_cast<uintptr_t>(tlut) & 3u) || (reinterpret_cast<uintptr_t>(out) & 3u))
     return QTIP_E_ALIGN;
-  DeviceInfo& di = device_info();
-  if (!di.ok) return (int)hipErrorInvalidDevice;
+  if (!device_info().ok) return (int)hipErrorInvalidDevice;
   hipError_t e = setup_once();
-  if (e != hipSuccess) return (int)e;
+  return e == hipSuccess ? QTIP_OK : (int)e;
+}
+
+int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x_f16,
+                                 const void* tlut, int m, int k, int bits, int nparts,
+                                 void* stream) {
+  int rc = check_matvec(parts, packed, x_f16, tlut, m, k, bits);
+  if (rc) return rc;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > ((((k >> 5) + 3) >> 2))) return QTIP_E_SHAPE;
+  return launch_matvec(parts, packed, x_f16, tlut, m, k, bits, nparts, (hipStream_t)stream);
+}
+
+int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,
+                           int m, int k, int bits, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits);
+  if (rc) return rc;
   int S = 1;
-  float* ws = nullptr;
-  unsigned* counters = nullptr;
   if (workspace) {
-    if (workspace_bytes < qtip_matvec_workspace_bytes(m, k, bits)) return QTIP_E_WORKSPACE;
+    S = choose_split(m, k, bits, device_info().cus);
+    if (S > 1 && workspace_bytes < (size_t)S * m * sizeof(float)) return QTIP_E_WORKSPACE;
     if (!aligned16(workspace)) return QTIP_E_ALIGN;
-    S = choose_split(m, k, bits, di.cus);
-    if ((size_t)(m >> 5) * sizeof(unsigned) > kCounterBytes) return QTIP_E_SHAPE;
-    counters = (unsigned*)workspace;
-    ws = (float*)((uint8_t*)workspace + kCounterBytes);
   }
-  const long units = (long)(m >> 5) * S;
-  const int grid = (int)(units < di.cus ? units : di.cus);
   hipStream_t st = (hipStream_t)stream;
-  auto* p = (const uint8_t*)packed;
-  auto* xx = (const uint16_t*)x_f16;
-  auto* t = (const uint32_t*)tlut;
-  switch (bits) {
-    case 2: matvec_kernel<2, 4><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
-    case 3: matvec_kernel<3, 3><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
-    default: matvec_kernel<4, 2><<<grid, kThreads, kMatvecLds, st>>>(out, p, xx, t, m, k, S, ws, counters); break;
-  }
+  if (S == 1) return launch_matvec(out, packed, x_f16, tlut, m, k, bits, 1, st);
+  rc = launch_matvec((float*)workspace, packed, x_f16, tlut, m, k, bits, S, st);
+  if (rc) return rc;
+  sum_parts_kernel<<<(m + 255) / 256, 256, 0, st>>>(out, (const float*)workspace, m, S);
   return (int)hipGetLastError();
 }
 

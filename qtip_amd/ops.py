@@ -14,18 +14,32 @@ from ._lib import QTIP_F16, QTIP_F32, check, lib, require_cuda, stream_ptr
 
 _DT = {torch.float16: QTIP_F16, torch.float32: QTIP_F32}
 
-# per-device scratch for the split-k matvec (zero-filled once, self-cleaning)
+# per-device scratch for the partial sums of the split-k matvec
 _WORKSPACE = {}
 _WORKSPACE_BYTES = 8 << 20
+_SPLIT = {}
 
 
 def _workspace(device, need):
     key = device.index if device.index is not None else torch.cuda.current_device()
     ws = _WORKSPACE.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, _WORKSPACE_BYTES), dtype=torch.uint8, device=device)
+        ws = torch.empty(max(need, _WORKSPACE_BYTES), dtype=torch.uint8, device=device)
         _WORKSPACE[key] = ws
     return ws
+
+
+def matvec_split(m, k, bits, device):
+    """Number of k splits the matvec kernel uses for this shape (cached per device)."""
+    key = (m, k, bits, device.index)
+    s = _SPLIT.get(key)
+    if s is None:
+        with torch.cuda.device(device):
+            s = lib().qtip_matvec_split(m, k, bits)
+        if s < 1:
+            raise ValueError(f"unsupported matvec shape {m}x{k} at {bits} bits")
+        _SPLIT[key] = s
+    return s
 
 
 def _ptr(t):
@@ -76,9 +90,8 @@ def decompress_matvec(packed, x, tlut, m, k, bits, out=None, split_k=True):
         if out.numel() != m:
             raise ValueError(f"out must hold {m} fp32 values")
     L = lib()
-    if split_k:
-        need = L.qtip_matvec_workspace_bytes(m, k, bits)
-        ws = _workspace(packed.device, need)
+    if split_k and matvec_split(m, k, bits, packed.device) > 1:
+        ws = _workspace(packed.device, 16 * m * 4)
         wsp, wsb = _ptr(ws), ws.numel()
     else:
         wsp, wsb = ctypes.c_void_p(0), 0
@@ -86,6 +99,22 @@ def decompress_matvec(packed, x, tlut, m, k, bits, out=None, split_k=True):
         check(L.qtip_decompress_matvec(_ptr(out), _ptr(packed), _ptr(x), _ptr(tlut), m, k, bits, wsp, wsb,
                                        stream_ptr(packed.device)), "qtip_decompress_matvec")
     return out
+
+
+def decompress_matvec_parts(packed, x, tlut, m, k, bits):
+    """(S, m) fp32 partial sums of decode(packed) @ x over S ranges of k; their
+    sum over axis 0 (in order) is the matvec.  S = matvec_split(...)."""
+    _check_packed(packed, m, k, bits)
+    _check_tlut(tlut, packed.device)
+    require_cuda(x, "x", torch.float16)
+    if x.numel() != k or x.device != packed.device:
+        raise ValueError(f"x must hold {k} fp16 values on {packed.device}")
+    S = matvec_split(m, k, bits, packed.device)
+    parts = torch.empty((S, m), dtype=torch.float32, device=packed.device)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_decompress_matvec_parts(_ptr(parts), _ptr(packed), _ptr(x), _ptr(tlut), m, k, bits, S,
+                                                 stream_ptr(packed.device)), "qtip_decompress_matvec_parts")
+    return parts
 
 
 def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):

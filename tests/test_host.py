@@ -44,7 +44,9 @@ def test_argument_rejection_without_gpu():
     assert L.qtip_rht(p, 0, p, 0, 1, 1, 100, 1, null, null, null, 1.0, null) == -1  # not a power of two
     assert L.qtip_rht(p, 0, p, 0, 1, 1, 12 * 64, 12, null, null, null, 1.0, null) == -2  # table missing
     assert L.qtip_rht(p, 7, p, 0, 1, 1, 64, 1, null, null, null, 1.0, null) == -5
-    assert L.qtip_matvec_workspace_bytes(4096, 4096, 2) >= 16 * 4096 * 4
+    assert L.qtip_matvec_split(33, 64, 2) == 0 and L.qtip_matvec_split(64, 64, 7) == 0
+    assert L.qtip_decompress_matvec_parts(p, p, p, p, 64, 64, 2, 0, null) in (-1, 100, 101)  # bad nparts (or no device)
+    assert L.qtip_decompress_matvec_parts(null, p, p, p, 64, 64, 2, 1, null) == -2
 
 
 def test_cpu_tensors_raise():
