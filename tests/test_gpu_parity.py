@@ -137,7 +137,7 @@ def test_gemm_vs_oracle(K, shape, batch):
     assert np.array_equal(got16, got.astype(np.float16).astype(np.float32))
 
 
-@pytest.mark.parametrize("n", [64, 256, 1024, 4096, 8192, 32768])
+@pytest.mark.parametrize("n", [2, 16, 64, 128, 256, 1024, 4096, 8192, 32768, 131072])
 @pytest.mark.parametrize("rows", [1, 3])
 def test_rht_pow2(n, rows):
     import qtip_amd.utils.matmul_had  # registers hadamard::hadamard
