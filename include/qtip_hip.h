@@ -103,9 +103,10 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16,
  *   in_dtype/out_dtype  QTIP_F16 or QTIP_F32
  *   pre   fp16[n] or NULL (input sign vector SU)
  *   post  fp32[n] or NULL (output scale vector SV)
- *   had_bits  order*order sign bits, bit (i*order+j) of a little-endian
- *             uint32 array set when H[i][j] == -1, already transposed by the
- *             caller for the "Ut" form; ignored (may be NULL) when order == 1
+ *   had_bits  order*order sign bits, column-major: bit (j*order+i) of a
+ *             little-endian uint32 array is set when H[i][j] == -1 (H already
+ *             transposed by the caller for the "Ut" form); ignored (may be
+ *             NULL) when order == 1
  *   in_parts  > 1: `in` holds in_parts arrays of rows*n elements that are
  *             summed on load (split-k partial sums); normally 1.
  * Replaces matmul_hadU_cuda / matmul_hadUt_cuda and the hadamard::hadamard
@@ -115,6 +116,32 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16,
 int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_parts,
              int rows, int n, int order, const uint32_t* had_bits,
              const void* pre_f16, const float* post_f32, float scale, void* stream);
+
+/* qtip_rht with the element-wise work of the layers around a QTIP linear folded in
+ * (used by the end-to-end decode loop; each mode cites what it replaces):
+ *   pre_mode 0  none
+ *   pre_mode 1  RMSNorm of the input row: fp16(w * fp16(x * rsqrt(mean(x^2) + eps)))
+ *               (model/llama.py:129-135); needs norm_weight_f16[n], in must be fp16
+ *   pre_mode 2  SiLU-gated product: row of `in` is [gate(n) | up(n)], the transform input is
+ *               fp16(fp16(silu(gate)) * up) (model/llama.py:399-400)
+ *   residual_f16 != NULL: out = fp16(residual + fp16(result)), the decoder layer's
+ *               residual addition (model/llama.py:964,979); out_dtype must be QTIP_F16.
+ * in_parts > 1 is only allowed with pre_mode 0. */
+int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int in_parts,
+                   int rows, int n, int order, const uint32_t* had_bits,
+                   const void* pre_f16, const float* post_f32, float scale,
+                   int pre_mode, const void* norm_weight_f16, float eps,
+                   const void* residual_f16, void* stream);
+
+/* Single-token decode attention for the end-to-end loop, one launch: rotary embedding of q and
+ * k in fp16 arithmetic (model/llama.py:264-295), write of k and v into the static cache at the
+ * token's position (model/cache_utils.py:1173-1193), softmax(q K^T / sqrt(d)) V over cache slots
+ * 0..pos (model/llama.py:866-880).  qkv_f16 = [heads*d | kv_heads*d | kv_heads*d] of the new token,
+ * caches are [kv_heads][max_len][d] fp16, pos_i64 points to the position in DEVICE memory (a
+ * recorded graph then follows the position), inv_freq[d/2] fp32.  out_f16 = [heads*d]. */
+int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16, void* v_cache_f16,
+                          const void* pos_i64, const float* inv_freq, int heads, int kv_heads,
+                          int head_dim, int max_len, void* stream);
 
 #ifdef __cplusplus
 }

@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -35,6 +35,11 @@ _SIGNATURES = {
     "qtip_rht": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                 ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                 ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p]),
+    "qtip_rht_fused": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_float,
+                                      ctypes.c_void_p, ctypes.c_void_p]),
+    "qtip_decode_attention": (ctypes.c_int, [ctypes.c_void_p] * 6 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -4,7 +4,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "csrc", "qtip_hip.hip")
+SRCS = [os.path.join(HERE, "csrc", f) for f in ("qtip_hip.hip", "qtip_rht.hip", "qtip_decoder.hip")]
 OUT = os.path.join(HERE, "libqtip_hip.so")
 
 # packed fp32 VALU forms are switched off for every HIP translation unit
@@ -16,7 +16,7 @@ HIPCC_FLAGS = [
 
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + [SRC, "-o", OUT + ".tmp"]
+    cmd = [hipcc] + HIPCC_FLAGS + SRCS + ["-o", OUT + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

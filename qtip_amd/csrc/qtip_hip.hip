@@ -419,144 +419,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// randomised Hadamard transform
-// ---------------------------------------------------------------------------
-// out = post * scale * (H_order (x) H_A (x) H_pp) (pre * in), n = order * A * pp.
-// The power-of-two part is split as H_A (x) H_pp (Sylvester matrices factor
-// that way) so that OT = order * A workgroups share one vector: workgroup
-// (iK, iA) produces the pp outputs of its row of the (order*A)-wide mix,
-//   z[c] = sum_{jK,jA} (-1)^(bits[iK][jK] + popcount(iA & jA)) v[(jK*A + jA)*pp + c],
-// followed by a pp-point Walsh-Hadamard transform of z.  All of a thread's
-// loads are issued before the first use (the transform is latency-bound: a
-// few KB per vector), the pp-point transform runs on cross-lane exchanges
-// inside a wave for the low six index bits and needs one LDS transposition
-// for the rest.
-constexpr int kRhtThreads = 1024;
-
-template <typename T>
-__device__ __forceinline__ float load_as_float(const T* p, size_t i);
-template <>
-__device__ __forceinline__ float load_as_float<float>(const float* p, size_t i) {
-  return p[i];
-}
-template <>
-__device__ __forceinline__ float load_as_float<_Float16>(const _Float16* p, size_t i) {
-  return (float)p[i];
-}
-
-// value of lane ^ (1 << b) for b = 0..5
-__device__ __forceinline__ float lane_xor(float v, int b) {
-  const int u = __builtin_bit_cast(int, v);
-  int r;
-  switch (b) {
-    case 0: r = __builtin_amdgcn_update_dpp(0, u, 0xB1, 0xF, 0xF, false); break;  // quad_perm 1,0,3,2
-    case 1: r = __builtin_amdgcn_update_dpp(0, u, 0x4E, 0xF, 0xF, false); break;  // quad_perm 2,3,0,1
-    case 2: r = __builtin_amdgcn_ds_swizzle(u, 0x101F); break;                    // xor 4
-    case 3: r = __builtin_amdgcn_ds_swizzle(u, 0x201F); break;                    // xor 8
-    case 4: r = __builtin_amdgcn_ds_swizzle(u, 0x401F); break;                    // xor 16
-    default: {
-      auto sw = __builtin_amdgcn_permlane32_swap((uint32_t)u, (uint32_t)u, false, false);
-      r = (int)((threadIdx.x & 32) ? sw[0] : sw[1]);
-    }
-  }
-  return __builtin_bit_cast(float, r);
-}
-
-// Walsh-Hadamard butterflies over lane bits 0 .. nbits-1 (natural order)
-__device__ __forceinline__ float wht_lanes(float v, int nbits, int lane) {
-#pragma unroll
-  for (int b = 0; b < 6; ++b) {
-    if (b < nbits) {
-      const float o = lane_xor(v, b);
-      v = ((lane >> b) & 1) ? o - v : v + o;
-    }
-  }
-  return v;
-}
-
-template <typename TIn, typename TOut, int CHUNK>
-__global__ __launch_bounds__(kRhtThreads) void rht_kernel(
-    TOut* __restrict__ out, const TIn* __restrict__ in, int in_parts, size_t part_stride, int n,
-    int order, int A, int pp, const uint32_t* __restrict__ had_bits,
-    const _Float16* __restrict__ pre, const float* __restrict__ post, float scale) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  float* red = reinterpret_cast<float*>(smem);  // [kRhtThreads] partial sums, then [pp] exchange
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int iK = blockIdx.x / A, iA = blockIdx.x - iK * A;
-  const size_t r = blockIdx.y;
-  const TIn* src = in + r * (size_t)n;
-  const int OT = order * A;
-  const int C = pp < kRhtThreads ? pp : kRhtThreads;  // pp <= kRhtThreads (launcher)
-  const int JG = kRhtThreads / C;
-  const int c = tid % C, jg = tid / C;
-
-  // ---- mix: z = sum over j = jg, jg+JG, ... of +-v[j*pp + c]
-  float z = 0.f;
-  for (int j0 = jg; j0 < OT; j0 += JG * CHUNK) {
-    float v[CHUNK];
-    uint32_t sg[CHUNK];
-#pragma unroll
-    for (int q = 0; q < CHUNK; ++q) {
-      const int j = j0 + q * JG;
-      v[q] = 0.f;
-      sg[q] = 0;
-      if (j < OT) {
-        const size_t idx = (size_t)j * pp + c;
-        float x = load_as_float<TIn>(src, idx);
-        for (int w = 1; w < in_parts; ++w) x += load_as_float<TIn>(src + w * part_stride, idx);
-        if (pre) x *= (float)pre[idx];
-        const int jK = j / A, jA = j - jK * A;
-        uint32_t neg = (uint32_t)__builtin_popcount(iA & jA);
-        if (order > 1) {
-          const unsigned bit = (unsigned)iK * order + jK;
-          neg += had_bits[bit >> 5] >> (bit & 31);
-        }
-        v[q] = x;
-        sg[q] = neg << 31;
-      }
-    }
-#pragma unroll
-    for (int q = 0; q < CHUNK; ++q) z += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[q]) ^ sg[q]);
-  }
-  if (JG > 1) {
-    red[tid] = z;
-    __syncthreads();
-    if (jg == 0)
-      for (int q = 1; q < JG; ++q) z += red[q * C + c];
-    __syncthreads();
-  }
-  // ---- pp-point transform: threads 0..pp-1 hold z[c] (c = low bits of the lane index)
-  const int W = pp > 64 ? pp >> 6 : 1;  // waves holding data
-  int nb0 = 0;
-  while (nb0 < 6 && (1 << nb0) < pp) ++nb0;
-  int cfin = c;
-  if (tid < pp) {
-    z = wht_lanes(z, nb0, lane);
-    if (W > 1) red[c] = z;
-  }
-  if (W > 1) {
-    __syncthreads();
-    if (tid < pp) {
-      // transposed read: the wave index of the element becomes the low lane bits
-      const int wv = tid >> 6;
-      const int ew = lane & (W - 1);                       // wave part of the element index
-      const int el = (lane / W) + (64 / W) * wv;           // lane part of the element index
-      cfin = 64 * ew + el;
-      z = red[cfin];
-      int nb = 0;
-      while ((1 << nb) < W) ++nb;
-      z = wht_lanes(z, nb, lane);
-    }
-  }
-  if (tid < pp) {
-    const size_t idx = (size_t)blockIdx.x * pp + cfin;
-    float y = z * scale;
-    if (post) y *= post[idx];
-    out[r * (size_t)n + idx] = (TOut)y;
-  }
-}
-
-// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 struct DeviceInfo {
@@ -651,7 +513,7 @@ int choose_split(int m, int k, int bits, int cus) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 2; }
+int qtip_abi_version(void) { return 3; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -800,57 +662,6 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
     if (le != hipSuccess) return (int)le;
   }
   return QTIP_OK;
-}
-
-int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
-             int order, const uint32_t* had_bits, const void* pre_f16, const float* post_f32,
-             float scale, void* stream) {
-  if (!out || !in) return QTIP_E_NULL;
-  if (rows < 1 || rows > 65535 || n < 1 || order < 1 || in_parts < 1 || in_parts > kMaxSplit)
-    return QTIP_E_SHAPE;
-  if (n % order) return QTIP_E_SHAPE;
-  const int p = n / order;
-  if (p & (p - 1)) return QTIP_E_SHAPE;
-  if (order > 1 && !had_bits) return QTIP_E_NULL;
-  if ((unsigned)out_dtype > 1u || (unsigned)in_dtype > 1u) return QTIP_E_DTYPE;
-  // split the power-of-two part: pp points per workgroup (64..1024), A row
-  // groups.  Every workgroup reads the whole vector (n / 1024 loads per
-  // thread whatever the split), so A only trades L2 traffic (order*A*n
-  // elements) against the size of the in-workgroup transform: go up to 64
-  // workgroups per vector.
-  int pp = p, A = 1;
-  while (pp > kRhtThreads) {
-    pp >>= 1;
-    A <<= 1;
-  }
-  while (pp > 64 && (long)order * A * 2 <= 64) {
-    pp >>= 1;
-    A <<= 1;
-  }
-  const long OT = (long)order * A;
-  const int JG = kRhtThreads / pp;
-  const long loads = (OT + JG - 1) / JG;
-  if (loads > 4096) return QTIP_E_SHAPE;
-  const size_t lds = kRhtThreads * sizeof(float);
-  dim3 grid((unsigned)OT, rows);
-  hipStream_t st = (hipStream_t)stream;
-  const size_t part_stride = (size_t)rows * n;
-  const _Float16* pre = (const _Float16*)pre_f16;
-#define QTIP_RHT(TI, TO)                                                                        \
-  if (loads > 8)                                                                                \
-    rht_kernel<TI, TO, 16><<<grid, kRhtThreads, lds, st>>>((TO*)out, (const TI*)in, in_parts,    \
-                                                           part_stride, n, order, A, pp,        \
-                                                           had_bits, pre, post_f32, scale);     \
-  else                                                                                          \
-    rht_kernel<TI, TO, 8><<<grid, kRhtThreads, lds, st>>>((TO*)out, (const TI*)in, in_parts,     \
-                                                          part_stride, n, order, A, pp,         \
-                                                          had_bits, pre, post_f32, scale)
-  if (in_dtype == QTIP_F16 && out_dtype == QTIP_F16) QTIP_RHT(_Float16, _Float16);
-  else if (in_dtype == QTIP_F16 && out_dtype == QTIP_F32) QTIP_RHT(_Float16, float);
-  else if (in_dtype == QTIP_F32 && out_dtype == QTIP_F16) QTIP_RHT(float, _Float16);
-  else QTIP_RHT(float, float);
-#undef QTIP_RHT
-  return (int)hipGetLastError();
 }
 
 }  // extern "C"

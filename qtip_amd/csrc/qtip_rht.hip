@@ -1,0 +1,342 @@
+// Randomised Hadamard transform kernel and its launchers (qtip_rht,
+// qtip_rht_fused).  Declarations: include/qtip_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qtip_hip.h"
+
+namespace {
+
+constexpr int kRhtThreads = 1024;
+constexpr int kMaxParts = 16;
+
+// out = post * scale * (H_order (x) H_A (x) H_pp) (pre * f(in)) [+ residual],  n = order * A * pp.
+// The power-of-two part is split as H_A (x) H_pp (Sylvester matrices factor
+// that way) so that OT = order * A workgroups share one vector: workgroup
+// (iK, iA) produces the pp outputs of its row of the (order*A)-wide mix,
+//   z[c] = sum_{jK,jA} (-1)^(bits[iK][jK] + popcount(iA & jA)) v[(jK*A + jA)*pp + c],
+// followed by a pp-point Walsh-Hadamard transform of z.  The transform is
+// latency-bound (a vector is a few KB), so every thread issues all of its
+// loads (n / 1024 elements and their companions) before the first use; the
+// pp-point transform runs on cross-lane exchanges inside a wave for the low
+// six index bits and needs one LDS transposition for the rest.
+//
+// Optional element-wise prologue f (what the layers around a QTIP linear do
+// to its input) and epilogue:
+//   PRE_RMSNORM   f(x) = fp16(w * fp16(x * rsqrt(mean(x^2) + eps)))   (model/llama.py:129-135)
+//   PRE_SILU_MUL  f = fp16(fp16(silu(g)) * u), g = in[i], u = in[n + i] (model/llama.py:399-400)
+//   residual      out = fp16(residual + fp16(result))                 (model/llama.py:964,979)
+enum { PRE_NONE = 0, PRE_RMSNORM = 1, PRE_SILU_MUL = 2 };
+
+struct RhtParams {
+  void* out;
+  const void* in;
+  const uint32_t* had_bits;
+  const _Float16* pre;       // SU or null
+  const float* post;         // SV or null
+  const _Float16* norm_w;    // PRE_RMSNORM weight
+  const _Float16* residual;  // or null
+  size_t part_stride;
+  size_t in_row_stride;      // elements between consecutive rows of `in`
+  float scale, eps;
+  int in_parts, n, order, logA, pp, pre_mode;
+};
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* p, size_t i);
+template <>
+__device__ __forceinline__ float ldf<float>(const float* p, size_t i) {
+  return p[i];
+}
+template <>
+__device__ __forceinline__ float ldf<_Float16>(const _Float16* p, size_t i) {
+  return (float)p[i];
+}
+
+// value of lane ^ (1 << b) for b = 0..5
+__device__ __forceinline__ float lane_xor(float v, int b) {
+  const int u = __builtin_bit_cast(int, v);
+  int r;
+  switch (b) {
+    case 0: r = __builtin_amdgcn_update_dpp(0, u, 0xB1, 0xF, 0xF, false); break;  // quad_perm 1,0,3,2
+    case 1: r = __builtin_amdgcn_update_dpp(0, u, 0x4E, 0xF, 0xF, false); break;  // quad_perm 2,3,0,1
+    case 2: r = __builtin_amdgcn_ds_swizzle(u, 0x101F); break;                    // xor 4
+    case 3: r = __builtin_amdgcn_ds_swizzle(u, 0x201F); break;                    // xor 8
+    case 4: r = __builtin_amdgcn_ds_swizzle(u, 0x401F); break;                    // xor 16
+    default: {
+      auto sw = __builtin_amdgcn_permlane32_swap((uint32_t)u, (uint32_t)u, false, false);
+      r = (int)((threadIdx.x & 32) ? sw[0] : sw[1]);
+    }
+  }
+  return __builtin_bit_cast(float, r);
+}
+
+// Walsh-Hadamard butterflies over lane bits 0 .. nbits-1 (natural order)
+__device__ __forceinline__ float wht_lanes(float v, int nbits, int lane) {
+#pragma unroll
+  for (int b = 0; b < 6; ++b) {
+    if (b < nbits) {
+      const float o = lane_xor(v, b);
+      v = ((lane >> b) & 1) ? o - v : v + o;
+    }
+  }
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int b = 0; b < 6; ++b) v += lane_xor(v, b);
+  return v;
+}
+
+// CH = loads in flight per thread and pass; FUSED enables the prologue modes
+// (which need the raw elements of the whole row, so the row must fit one pass);
+// RI = rows iK of the order-wide mix one workgroup produces (the loaded
+// elements are reused for all of them, which divides the load traffic of the
+// large table orders by RI).  Sign bits are indexed [jK][iK] so that the RI
+// signs of one element are adjacent bits of one word.
+template <typename TIn, typename TOut, int CH, bool FUSED, int RI>
+__global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
+  __shared__ float red[RI][kRhtThreads];  // partial sums, then the exchange buffer of the transform
+  __shared__ float wsum[16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int A = 1 << P.logA;
+  // blockIdx.x = (iK / RI) * A + iA   (RI > 1 only with A == 1)
+  const int iK0 = (blockIdx.x >> P.logA) * RI, iA = blockIdx.x & (A - 1);
+  const size_t r = blockIdx.y;
+  const int n = P.n, pp = P.pp, order = P.order;
+  const TIn* src = reinterpret_cast<const TIn*>(P.in) + r * P.in_row_stride;
+  const int OT = order << P.logA;
+  const int C = pp < kRhtThreads ? pp : kRhtThreads;  // pp <= kRhtThreads (launcher)
+  const int JG = kRhtThreads / C;
+  const int c = tid % C, jg = tid / C;
+  const int pre_mode = FUSED ? P.pre_mode : PRE_NONE;
+
+  float z[RI];
+#pragma unroll
+  for (int ri = 0; ri < RI; ++ri) z[ri] = 0.f;
+  const int npass = ((OT + JG - 1) / JG + CH - 1) / CH;  // the same for every thread (barriers inside)
+  for (int pass = 0; pass < npass; ++pass) {
+    const int j0 = jg + pass * JG * CH;
+    // ---- all loads of this pass: elements j = j0, j0+JG, ... of column c
+    float v[CH], f[CH], aux[FUSED ? CH : 1];
+    uint32_t sg[CH];
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      v[q] = 0.f;
+      f[q] = 0.f;
+      sg[q] = 0;
+      if (FUSED) aux[q] = 0.f;
+      if (j < OT) {
+        const size_t idx = (size_t)j * pp + c;
+        float x = ldf<TIn>(src, idx);
+        for (int w = 1; w < P.in_parts; ++w) x += ldf<TIn>(src + w * P.part_stride, idx);
+        v[q] = x;
+        if (FUSED && pre_mode == PRE_RMSNORM) aux[q] = (float)P.norm_w[idx];
+        if (FUSED && pre_mode == PRE_SILU_MUL) aux[q] = ldf<TIn>(src, (size_t)n + idx);
+        f[q] = P.pre ? (float)P.pre[idx] : 1.f;
+        const int jK = j >> P.logA, jA = j & (A - 1);
+        uint32_t neg = (uint32_t)__builtin_popcount(iA & jA) & 1u;
+        if (order > 1) {
+          const unsigned bit = (unsigned)jK * order + iK0;
+          neg ^= P.had_bits[bit >> 5] >> (bit & 31);  // bits 0..RI-1: rows iK0 .. iK0+RI-1
+        }
+        sg[q] = neg;
+      }
+    }
+    // ---- element-wise prologue
+    if (FUSED && pre_mode == PRE_RMSNORM) {
+      float ss = 0.f;
+#pragma unroll
+      for (int q = 0; q < CH; ++q) ss += v[q] * v[q];
+      ss = wave_sum(ss);
+      if (lane == 0) wsum[tid >> 6] = ss;
+      __syncthreads();
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) tot += wsum[w];
+      const float rs = __builtin_amdgcn_rsqf(tot / (float)n + P.eps);
+#pragma unroll
+      for (int q = 0; q < CH; ++q) v[q] = (float)(_Float16)(aux[q] * (float)(_Float16)(v[q] * rs));
+    } else if (FUSED && pre_mode == PRE_SILU_MUL) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        const float g = v[q];
+        const float sl = (float)(_Float16)(g / (1.f + __expf(-g)));
+        v[q] = (float)(_Float16)(sl * aux[q]);
+      }
+    }
+    // ---- mix
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const uint32_t vf = __builtin_bit_cast(uint32_t, v[q] * f[q]);
+#pragma unroll
+      for (int ri = 0; ri < RI; ++ri) z[ri] += __builtin_bit_cast(float, vf ^ ((sg[q] >> ri) << 31));
+    }
+  }
+  if (JG > 1) {
+#pragma unroll
+    for (int ri = 0; ri < RI; ++ri) red[ri][tid] = z[ri];
+    __syncthreads();
+  }
+  // ---- thread t < RI*pp takes row t / pp, column t % pp
+  const int row = tid / pp, col = tid - row * pp;  // col keeps the lane index in its low bits
+  const bool active = tid < RI * pp;
+  float y = 0.f;
+  if (active) {
+    if (JG > 1) {
+      for (int q = 0; q < JG; ++q) y += red[row][q * C + col];
+    } else {
+      y = z[0];  // JG == 1 implies pp == 1024 and RI == 1
+    }
+  }
+  if (JG > 1) __syncthreads();
+  // ---- pp-point transform
+  const int W = pp > 64 ? pp >> 6 : 1;  // waves holding one row
+  int nb0 = 0;
+  while (nb0 < 6 && (1 << nb0) < pp) ++nb0;
+  int cfin = col;
+  if (active) {
+    y = wht_lanes(y, nb0, lane);
+    if (W > 1) red[row][col] = y;
+  }
+  if (W > 1) {
+    __syncthreads();
+    if (active) {
+      // transposed read: the wave index of the element becomes the low lane bits
+      const int wv = col >> 6;
+      const int ew = lane & (W - 1);              // wave part of the element index
+      const int el = (lane / W) + (64 / W) * wv;  // lane part of the element index
+      cfin = 64 * ew + el;
+      y = red[row][cfin];
+      int nb = 0;
+      while ((1 << nb) < W) ++nb;
+      y = wht_lanes(y, nb, lane);
+    }
+  }
+  if (active) {
+    const size_t idx = ((size_t)(iK0 + row) * A + iA) * pp + cfin;
+    float o = y * P.scale;
+    if (P.post) o *= P.post[idx];
+    TOut* op = reinterpret_cast<TOut*>(P.out) + r * (size_t)n + idx;
+    if (FUSED && P.residual) {
+      const float res = (float)P.residual[r * (size_t)n + idx];
+      *op = (TOut)(_Float16)(res + (float)(_Float16)o);
+    } else {
+      *op = (TOut)o;
+    }
+  }
+}
+
+template <typename TI, typename TO, bool FUSED>
+int launch_rht_l(const RhtParams& P, dim3 grid, long loads, int ri, hipStream_t st) {
+  // a prologue needs the whole row in one pass
+  if (FUSED && P.pre_mode == PRE_RMSNORM && loads > 16) return QTIP_E_SHAPE;
+  if (ri == 4) {
+    if (loads <= 8) rht_kernel<TI, TO, 8, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(P);
+    else rht_kernel<TI, TO, 16, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(P);
+  } else {
+    if (loads <= 4) rht_kernel<TI, TO, 4, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
+    else if (loads <= 8) rht_kernel<TI, TO, 8, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
+    else rht_kernel<TI, TO, 16, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
+  }
+  return (int)hipGetLastError();
+}
+
+int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream) {
+  if (!P.out || !P.in) return QTIP_E_NULL;
+  const int n = P.n, order = P.order;
+  if (rows < 1 || rows > 65535 || n < 1 || order < 1 || P.in_parts < 1 || P.in_parts > kMaxParts)
+    return QTIP_E_SHAPE;
+  if (n % order) return QTIP_E_SHAPE;
+  const int p = n / order;
+  if (p & (p - 1)) return QTIP_E_SHAPE;
+  if (order > 1 && !P.had_bits) return QTIP_E_NULL;
+  if ((unsigned)out_dtype > 1u || (unsigned)in_dtype > 1u) return QTIP_E_DTYPE;
+  // split the power-of-two part: pp points per workgroup (<= 1024), A row
+  // groups.  Every workgroup reads the whole vector (n / 1024 loads per thread
+  // whatever the split), so A only trades L2 traffic (order*A*n elements)
+  // against the size of the in-workgroup transform: up to 64 workgroups per vector.
+  int pp = p, logA = 0;
+  while (pp > kRhtThreads) {
+    pp >>= 1;
+    ++logA;
+  }
+  while (pp > 64 && ((long)order << (logA + 1)) <= 64) {
+    pp >>= 1;
+    ++logA;
+  }
+  const long OT = (long)order << logA;
+  const int JG = kRhtThreads / pp;
+  const long loads = (OT + JG - 1) / JG;
+  P.logA = logA;
+  P.pp = pp;
+  // large table orders: four rows of the mix per workgroup
+  const int ri = (logA == 0 && order >= 64 && order % 4 == 0 && 4 * pp <= kRhtThreads && JG > 1) ? 4 : 1;
+  dim3 grid((unsigned)(OT / ri), rows);
+  hipStream_t st = (hipStream_t)stream;
+  const bool fused = P.pre_mode != PRE_NONE || P.residual != nullptr;
+  if (fused) {
+    // fused forms exist for the two combinations the decode loop uses
+    if (out_dtype != QTIP_F16) return QTIP_E_DTYPE;
+    if (in_dtype == QTIP_F16) return launch_rht_l<_Float16, _Float16, true>(P, grid, loads, ri, st);
+    return launch_rht_l<float, _Float16, true>(P, grid, loads, ri, st);
+  }
+  if (in_dtype == QTIP_F16 && out_dtype == QTIP_F16) return launch_rht_l<_Float16, _Float16, false>(P, grid, loads, ri, st);
+  if (in_dtype == QTIP_F16 && out_dtype == QTIP_F32) return launch_rht_l<_Float16, float, false>(P, grid, loads, ri, st);
+  if (in_dtype == QTIP_F32 && out_dtype == QTIP_F16) return launch_rht_l<float, _Float16, false>(P, grid, loads, ri, st);
+  return launch_rht_l<float, float, false>(P, grid, loads, ri, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
+             int order, const uint32_t* had_bits, const void* pre_f16, const float* post_f32,
+             float scale, void* stream) {
+  RhtParams P{};
+  P.out = out;
+  P.in = in;
+  P.had_bits = had_bits;
+  P.pre = (const _Float16*)pre_f16;
+  P.post = post_f32;
+  P.part_stride = (size_t)(rows > 0 ? rows : 0) * (size_t)(n > 0 ? n : 0);
+  P.in_row_stride = (size_t)(n > 0 ? n : 0);
+  P.scale = scale;
+  P.in_parts = in_parts;
+  P.n = n;
+  P.order = order;
+  P.pre_mode = PRE_NONE;
+  return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows,
+                   int n, int order, const uint32_t* had_bits, const void* pre_f16,
+                   const float* post_f32, float scale, int pre_mode, const void* norm_weight_f16,
+                   float eps, const void* residual_f16, void* stream) {
+  if (pre_mode < PRE_NONE || pre_mode > PRE_SILU_MUL) return QTIP_E_SHAPE;
+  if (pre_mode == PRE_RMSNORM && !norm_weight_f16) return QTIP_E_NULL;
+  if (pre_mode != PRE_NONE && in_parts != 1) return QTIP_E_SHAPE;
+  RhtParams P{};
+  P.out = out;
+  P.in = in;
+  P.had_bits = had_bits;
+  P.pre = (const _Float16*)pre_f16;
+  P.post = post_f32;
+  P.norm_w = (const _Float16*)norm_weight_f16;
+  P.residual = (const _Float16*)residual_f16;
+  P.part_stride = (size_t)(rows > 0 ? rows : 0) * (size_t)(n > 0 ? n : 0);
+  // gate and up halves sit side by side in a row of 2n elements
+  P.in_row_stride = (size_t)(n > 0 ? n : 0) * (pre_mode == PRE_SILU_MUL ? 2 : 1);
+  P.scale = scale;
+  P.eps = eps;
+  P.in_parts = in_parts;
+  P.n = n;
+  P.order = order;
+  P.pre_mode = pre_mode;
+  return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+}  // extern "C"

@@ -21,7 +21,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops
 from .linear.quantized_linear import QuantizedLinear
+from .utils.matmul_had import had_bits
 
 
 class LlamaConfig:
@@ -98,6 +100,44 @@ class DecoderLayer(nn.Module):
         x = x + self.down(F.silu(gate) * up)
         return x
 
+    def decode_fused(self, x, k_cache, v_cache, pos, inv_freq):
+        """One new token, x (1, hidden) fp16: 13 launches (4 x [transform, matvec, transform] + attention)."""
+        cfg = self.cfg
+        if not hasattr(self, "_fused"):
+            self._fused = [_FusedLinear(l) for l in (self.qkv, self.o, self.up_gate, self.down)]
+        qkv_l, o_l, ug_l, down_l = self._fused
+        qkv = qkv_l(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+        attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
+                                    cfg.head_dim)
+        x = o_l(attn.reshape(1, -1), residual=x)
+        ug = ug_l(x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+        return down_l(ug, ops.PRE_SILU_MUL, residual=x)
+
+
+class _FusedLinear:
+    """The three launches of a bs=1 QuantizedLinear with the neighbouring element-wise work of
+    the decoder layer folded into the two transforms (RMSNorm or SiLU*up on the way in, the
+    residual addition on the way out)."""
+
+    def __init__(self, lin):
+        dev = lin.trellis.device
+        self.lin = lin
+        self.n, self.m, self.K = lin.in_features, lin.out_features, lin.K
+        self.trellis = lin.trellis.reshape(-1)
+        self.tlut = lin.tlut.data.reshape(-1).contiguous()
+        self.SU, self.SV = lin.SU, lin.SV
+        self.Kl, self.Kr = lin.K_left, lin.K_right
+        self.bl = had_bits(lin.had_left, self.Kl, True, dev) if self.Kl > 1 else None
+        self.br = had_bits(lin.had_right, self.Kr, False, dev) if self.Kr > 1 else None
+
+    def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
+        xt = ops.rht(x, order=self.Kl, had_bits=self.bl, pre=self.SU, scale=(self.n**-0.5) / 32.0,
+                     out_dtype=torch.float16, pre_mode=pre_mode, norm_weight=norm_weight, eps=eps)
+        parts = ops.decompress_matvec_parts(self.trellis, xt.reshape(-1), self.tlut, self.m, self.n, self.K)
+        return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
+                       post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
+                       residual=residual)
+
 
 def _rotate_half(x):
     x1, x2 = x[..., :x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
@@ -139,9 +179,17 @@ class LlamaDecoder(nn.Module):
         x = self.norm(x)
         return (x @ self.lm_head.T).float()
 
+    def decode_fused(self, tok, pos):
+        """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab) fp32, fused kernels."""
+        x = self.embed[tok.reshape(-1)]
+        for i, layer in enumerate(self.layers):
+            x = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq)
+        x = self.norm(x)
+        return (x @ self.lm_head.T).float().reshape(1, 1, -1)
+
 
 @torch.no_grad()
-def generate(model, prompt_ids, max_new_tokens, use_graph=True):
+def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True):
     """Greedy decode.  Returns (token ids, decode seconds, tokens per second);
     throughput is max_new_tokens / decode wall-clock as in eval/interactive_gen.py:71-85."""
     dev = prompt_ids.device
@@ -153,7 +201,7 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True):
     out = [tok.clone()]
 
     def step():
-        lg = model(static_tok, static_pos)
+        lg = model.decode_fused(static_tok, static_pos) if fused else model(static_tok, static_pos)
         return lg[:, -1].argmax(-1, keepdim=True)
 
     graph = None

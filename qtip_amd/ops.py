@@ -134,16 +134,26 @@ def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     return out
 
 
-def rht(x, order=1, had_bits=None, pre=None, post=None, scale=None, out_dtype=None, in_parts=1):
-    """out[r] = post * scale * (H_order (x) H_p)(pre * x[r]) over the last axis.
+PRE_NONE, PRE_RMSNORM, PRE_SILU_MUL = 0, 1, 2
+
+
+def rht(x, order=1, had_bits=None, pre=None, post=None, scale=None, out_dtype=None, in_parts=1, pre_mode=PRE_NONE,
+        norm_weight=None, eps=0.0, residual=None):
+    """out[r] = post * scale * (H_order (x) H_p)(pre * f(x[r])) (+ residual) over the last axis.
 
     x: (..., n) fp16 or fp32 (with in_parts > 1: (in_parts, ..., n), summed on load).
-    had_bits: int32 device tensor of packed sign bits for order > 1.
-    scale defaults to n ** -0.5.
+    had_bits: int32 device tensor of packed sign bits for order > 1.  scale defaults to n ** -0.5.
+    pre_mode / norm_weight / eps / residual: element-wise work of the surrounding layer folded
+    into the same launch (see qtip_rht_fused in include/qtip_hip.h); with PRE_SILU_MUL the last
+    axis of x holds [gate | up] and n is half of it.
     """
     require_cuda(x, "x", (torch.float16, torch.float32))
     n = x.shape[-1]
-    rows = x.numel() // n // in_parts
+    if pre_mode == PRE_SILU_MUL:
+        if n % 2:
+            raise ValueError("gate|up input needs an even last dimension")
+        n //= 2
+    rows = x.numel() // x.shape[-1] // in_parts
     if n % order:
         raise ValueError(f"order {order} does not divide {n}")
     p = n // order
@@ -162,23 +172,65 @@ def rht(x, order=1, had_bits=None, pre=None, post=None, scale=None, out_dtype=No
         if post.numel() != n:
             raise ValueError(f"post must hold {n} values")
     out_dtype = out_dtype or x.dtype
-    shape = x.shape[1:] if in_parts > 1 else x.shape
+    shape = list(x.shape[1:] if in_parts > 1 else x.shape)
+    shape[-1] = n
+    fused = pre_mode != PRE_NONE or residual is not None
+    if pre_mode == PRE_RMSNORM:
+        require_cuda(norm_weight, "norm_weight", torch.float16)
+        if norm_weight.numel() != n or x.dtype != torch.float16:
+            raise ValueError("RMSNorm prologue needs an fp16 input and an fp16 weight of the same length")
+    if pre_mode not in (PRE_NONE, PRE_RMSNORM, PRE_SILU_MUL) or (pre_mode != PRE_NONE and in_parts != 1):
+        raise ValueError("bad pre_mode")
+    if residual is not None:
+        require_cuda(residual, "residual", torch.float16)
+        if out_dtype != torch.float16 or residual.numel() != rows * n:
+            raise ValueError("residual needs fp16 output and one value per output element")
     out = torch.empty(shape, dtype=out_dtype, device=x.device)
     if rows == 0:
         return out
     if scale is None:
         scale = n ** -0.5
+    L = lib()
     with torch.cuda.device(x.device):
-        # rows beyond the grid limit are processed in slices
-        xf = x.reshape(in_parts, rows, n) if in_parts > 1 else x.reshape(rows, n)
+        width = x.shape[-1]
+        xf = x.reshape(in_parts, rows, width) if in_parts > 1 else x.reshape(rows, width)
         of = out.reshape(rows, n)
+        rf = residual.reshape(rows, n) if residual is not None else None
         step = 65535 if in_parts == 1 else rows
         if in_parts > 1 and rows > 65535:
             raise ValueError("too many rows for a split input")
         for r0 in range(0, rows, step):
             r1 = min(rows, r0 + step)
             src = xf if in_parts > 1 else xf[r0:r1]
-            check(lib().qtip_rht(_ptr(of[r0:r1]), _DT[out_dtype], _ptr(src), _DT[x.dtype], in_parts, r1 - r0, n,
+            if fused:
+                check(L.qtip_rht_fused(_ptr(of[r0:r1]), _DT[out_dtype], _ptr(src), _DT[x.dtype], in_parts, r1 - r0, n,
+                                       order, _ptr(had_bits), _ptr(pre), _ptr(post), ctypes.c_float(scale), pre_mode,
+                                       _ptr(norm_weight), ctypes.c_float(eps),
+                                       _ptr(rf[r0:r1]) if rf is not None else _ptr(None),
+                                       stream_ptr(x.device)), "qtip_rht_fused")
+            else:
+                check(L.qtip_rht(_ptr(of[r0:r1]), _DT[out_dtype], _ptr(src), _DT[x.dtype], in_parts, r1 - r0, n,
                                  order, _ptr(had_bits), _ptr(pre), _ptr(post), ctypes.c_float(scale),
                                  stream_ptr(x.device)), "qtip_rht")
+    return out
+
+
+def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head_dim):
+    """Attention output (heads*head_dim,) fp16 of one new token: RoPE, cache write at `pos`
+    (device int64 tensor with one element) and attention over cache slots 0..pos in one launch.
+    k_cache / v_cache: (1, kv_heads, max_len, head_dim) fp16, updated in place."""
+    require_cuda(qkv, "qkv", torch.float16)
+    require_cuda(k_cache, "k_cache", torch.float16)
+    require_cuda(v_cache, "v_cache", torch.float16)
+    require_cuda(pos, "pos", torch.int64)
+    require_cuda(inv_freq, "inv_freq", torch.float32)
+    max_len = k_cache.shape[-2]
+    if qkv.numel() != (heads + 2 * kv_heads) * head_dim or k_cache.numel() != kv_heads * max_len * head_dim \
+            or v_cache.shape != k_cache.shape or inv_freq.numel() != head_dim // 2 or pos.numel() != 1:
+        raise ValueError("decode_attention: inconsistent shapes")
+    out = torch.empty(heads * head_dim, dtype=torch.float16, device=qkv.device)
+    with torch.cuda.device(qkv.device):
+        check(lib().qtip_decode_attention(_ptr(out), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos),
+                                          _ptr(inv_freq), heads, kv_heads, head_dim, max_len,
+                                          stream_ptr(qkv.device)), "qtip_decode_attention")
     return out

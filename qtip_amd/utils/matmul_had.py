@@ -50,8 +50,9 @@ def get_hadK(n, transpose=False):
 
 
 def _pack_bits(neg):
-    """(K, K) boolean array (True = -1) -> int32 words, bit i*K+j little-endian."""
-    flat = np.asarray(neg, dtype=np.uint8).reshape(-1)
+    """(K, K) boolean array neg[i][j] (True = -1) -> int32 words, column-major:
+    bit j*K+i (little-endian) holds neg[i][j], the layout the kernel reads."""
+    flat = np.ascontiguousarray(np.asarray(neg, dtype=np.uint8).T).reshape(-1)
     pad = (-flat.size) % 32
     flat = np.concatenate([flat, np.zeros(pad, dtype=np.uint8)])
     words = np.packbits(flat.reshape(-1, 8)[:, ::-1], axis=1).reshape(-1, 4)

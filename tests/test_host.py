@@ -134,7 +134,7 @@ def test_get_hadK_and_bits():
     w = mh._pack_bits(neg).view(np.uint32)
     for i in range(20):
         for j in range(20):
-            b = i * 20 + j
+            b = j * 20 + i
             assert ((w[b >> 5] >> (b & 31)) & 1) == neg[i, j]
 
 
