@@ -81,6 +81,7 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // decompress + matvec
 // ---------------------------------------------------------------------------
 constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
+constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a workgroup's k range
 
 // 32 states of one wave-load.  All hashes, addresses and the 32 table reads
 // are issued first and the 32 dot products follow, so a read has the rest of
@@ -92,6 +93,7 @@ __device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u
                                                   uint32_t slot4, float acc[4]) {
   uint32_t P[16], W[32];
   packed_states<K>(ld, P);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
@@ -177,13 +179,16 @@ __device__ __forceinline__ void load_x(const uint16_t* __restrict__ xw, uint32_t
 // across unit boundaries and every load in the loop is unconditional (a
 // conditional prefetch makes the compiler wait for it at once): padding items
 // fetch offset 0 and are skipped by the arithmetic.
-template <int K, int DEPTH>
+// XLDS: the x values of the workgroup's k range are staged in LDS once
+// (needs 256 bytes per wave-load of the range) and read from there.
+template <int K, int DEPTH, bool XLDS>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
     const uint32_t* __restrict__ tlut, int m, int k, int S, int wl_per) {
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
   float* part = reinterpret_cast<float*>(smem + kLut128Bytes);  // [2][kWaves][32]
+  uint8_t* xs_lds = smem + kLut128Bytes + 2 * kWaves * 32 * sizeof(float);  // [wl_per][256] when XLDS
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int a = lane & 15, g = lane >> 4;
@@ -221,14 +226,14 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   uint32_t l_rboff = (uint32_t)rb0 * rb_bytes;
   const uint32_t rb_step_bytes = (uint32_t)rb_step * rb_bytes;
   LaneData<K> buf[DEPTH];
-  u32x2 xbuf[DEPTH][4];
+  u32x2 xbuf[XLDS ? 1 : DEPTH][4];
   auto issue = [&](int d) {
     const bool valid = l_j < nvj && l_t < T;
     const uint32_t wl = (uint32_t)(w_first + l_j * kWaves);
     const uint32_t woff = valid ? l_rboff + wl * WL_BYTES : 0u;
     const uint32_t xw = valid ? wl * 256u : 0u;
     buf[d] = load_lane_buf<K>(rs_w, loff, woff);
-    load_x_buf(rs_x, xoff, xw, xbuf[d]);
+    if constexpr (!XLDS) load_x_buf(rs_x, xoff, xw, xbuf[d]);
     ++l_t;
     if (++l_j == npw) {
       l_j = 0;
@@ -240,7 +245,19 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   for (int d = 0; d < DEPTH; ++d) issue(d);
 
   build_lut128(lut, tlut, tid, kThreads);
+  if constexpr (XLDS) {
+    // x of wave-loads [wl0, wl1): 16 bytes per thread and pass
+    const int xbytes = (wl1 - wl0) * 256;
+    const int kbytes = k * 2;
+    for (int o = tid * 16; o < xbytes; o += kThreads * 16) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (wl0 * 256 + o < kbytes)
+        v = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(x) + (size_t)wl0 * 256 + o);
+      *reinterpret_cast<u32x4*>(xs_lds + o) = v;
+    }
+  }
   __syncthreads();
+  const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)wave * 256u;  // wave-load w_first
 
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   int parity = 0, c_j = 0, c_rb = rb0;
@@ -248,7 +265,18 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (t + d < T) {
-        if (c_j < nvj) matvec_accumulate<K>(buf[d], xbuf[d], slot4, acc);
+        if (c_j < nvj) {
+          if constexpr (XLDS) {
+            typedef __attribute__((address_space(3))) const u32x2 lds_u32x2_t;
+            u32x2 xv[4];
+            const uint32_t xa = xs_lane + (uint32_t)c_j * (kWaves * 256u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xv[q] = *(lds_u32x2_t*)(uintptr_t)(xa + 16u * q);
+            matvec_accumulate<K>(buf[d], xv, slot4, acc);
+          } else {
+            matvec_accumulate<K>(buf[d], xbuf[d], slot4, acc);
+          }
+        }
       }
       // the stage's registers are refilled only after their last use, so the
       // refill reuses them in place (no copies, no wait on the new load)
@@ -459,9 +487,12 @@ hipError_t setup_once() {
     QTIP_ALLOW((decode_kernel<2>), kLutBytes)
     QTIP_ALLOW((decode_kernel<3>), kLutBytes)
     QTIP_ALLOW((decode_kernel<4>), kLutBytes)
-    QTIP_ALLOW((matvec_kernel<2, 4>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<3, 3>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<4, 2>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<2, 4, false>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<3, 3, false>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 2>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 4>), kGemmLds)
@@ -575,10 +606,20 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   auto* p = (const uint8_t*)packed;
   auto* xx = (const uint16_t*)x_f16;
   auto* t = (const uint32_t*)tlut;
-  switch (bits) {
-    case 2: matvec_kernel<2, 4><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-    case 3: matvec_kernel<3, 3><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-    default: matvec_kernel<4, 2><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+  const size_t xbytes = (size_t)wl_per * 256;
+  if (xbytes <= kMatvecXBytes) {
+    const size_t lds = kMatvecLds + xbytes;
+    switch (bits) {
+      case 2: matvec_kernel<2, 6, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 3: matvec_kernel<3, 4, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      default: matvec_kernel<4, 3, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+    }
+  } else {
+    switch (bits) {
+      case 2: matvec_kernel<2, 4, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 3: matvec_kernel<3, 3, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      default: matvec_kernel<4, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+    }
   }
   return (int)hipGetLastError();
 }

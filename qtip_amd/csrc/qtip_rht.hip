@@ -118,32 +118,60 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
   const int npass = ((OT + JG - 1) / JG + CH - 1) / CH;  // the same for every thread (barriers inside)
   for (int pass = 0; pass < npass; ++pass) {
     const int j0 = jg + pass * JG * CH;
-    // ---- all loads of this pass: elements j = j0, j0+JG, ... of column c
+    // ---- all loads of this pass: elements j = j0, j0+JG, ... of column c.
+    // The loads are unconditional (out-of-range items re-read element c and are
+    // masked afterwards) and nothing depends on them until all are issued.
+    TIn xr[CH], ar[FUSED ? CH : 1];
+    float xs[CH];
+    _Float16 sr[CH];
+    uint32_t br[CH];
+    bool ok[CH];
+    size_t idx[CH];
+    // (one uniform branch per array, never per element: a load inside a
+    // per-element branch is waited for at once)
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      ok[q] = j < OT;
+      idx[q] = (size_t)(ok[q] ? j : 0) * pp + c;
+      xr[q] = src[idx[q]];
+      xs[q] = 0.f;
+      sr[q] = (_Float16)1.f;
+      br[q] = 0;
+    }
+    if (P.pre) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) sr[q] = P.pre[idx[q]];
+    }
+    if (order > 1) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        const int j = j0 + q * JG;
+        const unsigned bit = (unsigned)((ok[q] ? j : 0) >> P.logA) * order + iK0;
+        br[q] = P.had_bits[bit >> 5] >> (bit & 31);  // bits 0..RI-1: rows iK0 .. iK0+RI-1
+      }
+    }
+    if (FUSED && pre_mode == PRE_RMSNORM) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) ar[q] = (TIn)P.norm_w[idx[q]];
+    }
+    if (FUSED && pre_mode == PRE_SILU_MUL) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) ar[q] = src[(size_t)n + idx[q]];
+    }
+    for (int w = 1; w < P.in_parts; ++w) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) xs[q] += ldf<TIn>(src + w * P.part_stride, idx[q]);
+    }
     float v[CH], f[CH], aux[FUSED ? CH : 1];
     uint32_t sg[CH];
 #pragma unroll
     for (int q = 0; q < CH; ++q) {
       const int j = j0 + q * JG;
-      v[q] = 0.f;
-      f[q] = 0.f;
-      sg[q] = 0;
-      if (FUSED) aux[q] = 0.f;
-      if (j < OT) {
-        const size_t idx = (size_t)j * pp + c;
-        float x = ldf<TIn>(src, idx);
-        for (int w = 1; w < P.in_parts; ++w) x += ldf<TIn>(src + w * P.part_stride, idx);
-        v[q] = x;
-        if (FUSED && pre_mode == PRE_RMSNORM) aux[q] = (float)P.norm_w[idx];
-        if (FUSED && pre_mode == PRE_SILU_MUL) aux[q] = ldf<TIn>(src, (size_t)n + idx);
-        f[q] = P.pre ? (float)P.pre[idx] : 1.f;
-        const int jK = j >> P.logA, jA = j & (A - 1);
-        uint32_t neg = (uint32_t)__builtin_popcount(iA & jA) & 1u;
-        if (order > 1) {
-          const unsigned bit = (unsigned)jK * order + iK0;
-          neg ^= P.had_bits[bit >> 5] >> (bit & 31);  // bits 0..RI-1: rows iK0 .. iK0+RI-1
-        }
-        sg[q] = neg;
-      }
+      v[q] = ok[q] ? (float)xr[q] + xs[q] : 0.f;
+      if (FUSED) aux[q] = (float)ar[q];
+      f[q] = (float)sr[q];
+      sg[q] = br[q] ^ ((uint32_t)__builtin_popcount(iA & (j & (A - 1))) & 1u);
     }
     // ---- element-wise prologue
     if (FUSED && pre_mode == PRE_RMSNORM) {

@@ -277,3 +277,107 @@ def test_graph_capture_replays():
         torch.cuda.synchronize()
         assert torch.equal(static_out, ref), it
     assert torch.equal(layer(dev(L["x"]), *args), eager)
+
+
+# ---- fused transform prologues / epilogue and the decode attention kernel ----
+def _f16(a):
+    return np.asarray(a, dtype=np.float16)
+
+
+@pytest.mark.parametrize("n", [4096, 8192, 1024])
+def test_rht_fused_rmsnorm(n):
+    # fp16(w * fp16(x * rsqrt(mean(x^2) + eps))) (model/llama.py:129-135), then the input transform
+    from qtip_amd import ops
+    rng = np.random.default_rng(n)
+    x = _f16(rng.standard_normal((1, n)))
+    w = _f16(1 + 0.1 * rng.standard_normal(n))
+    su = _f16(np.sign(rng.standard_normal(n)))
+    eps = 1e-5
+    got = ops.rht(dev(x), pre=dev(su), scale=(n**-0.5) / 32, out_dtype=torch.float16, pre_mode=ops.PRE_RMSNORM,
+                  norm_weight=dev(w), eps=eps).cpu().numpy()
+    xf = x.astype(np.float32)
+    h = _f16(xf * (1.0 / np.sqrt((xf.astype(np.float64)**2).mean() + eps)).astype(np.float32))
+    normed = _f16(w.astype(np.float32) * h.astype(np.float32))
+    ref = O.hadamard_transform(normed.astype(np.float32) * su.astype(np.float32), transpose=True) / 32
+    assert_close(got, ref, 3e-3, 1e-3)
+
+
+def test_rht_fused_silu_mul_and_residual():
+    from qtip_amd import ops
+    from qtip_amd.utils import matmul_had as mh
+    n = 11008
+    rng = np.random.default_rng(1)
+    ug = _f16(rng.standard_normal((1, 2 * n)))
+    su = _f16(np.sign(rng.standard_normal(n)))
+    bits = mh.had_bits(None, 172, True, "cuda")
+    got = ops.rht(dev(ug), order=172, had_bits=bits, pre=dev(su), scale=(n**-0.5) / 32, out_dtype=torch.float16,
+                  pre_mode=ops.PRE_SILU_MUL).cpu().numpy()
+    g, u = ug[0, :n].astype(np.float32), ug[0, n:].astype(np.float32)
+    act = _f16(_f16(g / (1 + np.exp(-g))).astype(np.float32) * u)
+    ref = O.hadamard_transform(act.astype(np.float32)[None] * su.astype(np.float32), transpose=True) / 32
+    assert_close(got, ref, 3e-3, 1e-3)
+    # output transform with the residual addition folded in, from two split-k partial vectors
+    m = 4096
+    parts = rng.standard_normal((2, 1, m)).astype(np.float32)
+    sv = (rng.standard_normal(m) * 0.05).astype(np.float32)
+    res = _f16(rng.standard_normal((1, m)))
+    got = ops.rht(dev(parts), post=dev(sv), scale=(m**-0.5) * 32, out_dtype=torch.float16, in_parts=2,
+                  residual=dev(res)).cpu().numpy()
+    y = _f16(O.hadamard_transform(parts[0] + parts[1]) * 32 * sv)
+    ref = _f16(res.astype(np.float32) + y.astype(np.float32))
+    assert_close(got, ref, 3e-3, 1e-3)
+
+
+@pytest.mark.parametrize("heads,kv_heads,pos", [(32, 32, 0), (32, 32, 130), (32, 8, 77), (8, 8, 511)])
+def test_decode_attention(heads, kv_heads, pos):
+    # RoPE (model/llama.py:264-295) + cache write + attention over slots 0..pos, against torch in fp32
+    from qtip_amd import ops
+    D, max_len = 128, 512
+    g = torch.Generator().manual_seed(pos + heads)
+    qkv = torch.randn((heads + 2 * kv_heads) * D, generator=g).half().cuda()
+    kc = (torch.randn(1, kv_heads, max_len, D, generator=g) * 0.5).half().cuda()
+    vc = torch.randn(1, kv_heads, max_len, D, generator=g).half().cuda()
+    kc0, vc0 = kc.clone(), vc.clone()
+    inv_freq = (1.0 / (10000.0**(torch.arange(0, D, 2).float() / D))).cuda()
+    p = torch.tensor([pos], device="cuda")
+    out = ops.decode_attention(qkv, kc, vc, p, inv_freq, heads, kv_heads, D)
+    # reference
+    q = qkv[:heads * D].view(heads, D).float()
+    k = qkv[heads * D:(heads + kv_heads) * D].view(kv_heads, D).float()
+    v = qkv[(heads + kv_heads) * D:].view(kv_heads, D)
+    ang = pos * inv_freq
+    cos = torch.cat([ang.cos(), ang.cos()]).half().float()
+    sin = torch.cat([ang.sin(), ang.sin()]).half().float()
+
+    def rope(t):
+        rot = torch.cat([-t[:, D // 2:], t[:, :D // 2]], dim=1)
+        return ((t * cos).half().float() + (rot * sin).half().float()).half()
+
+    qe, ke = rope(q), rope(k)
+    kc0[0, :, pos] = ke
+    vc0[0, :, pos] = v
+    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)  # cache rows written exactly as the reference would
+    rep = heads // kv_heads
+    kk = kc0[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
+    vv = vc0[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
+    sc = torch.einsum("hd,htd->ht", qe.float(), kk) / D**0.5
+    ref = torch.einsum("ht,htd->hd", sc.softmax(-1), vv).reshape(-1)
+    assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
+
+
+def test_fused_decode_step_matches_generic():
+    # the 13-launch fused decode step against the module-by-module forward of the same model
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64)
+    ids = torch.randint(0, cfg.vocab, (1, 9), generator=torch.Generator().manual_seed(0)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(9, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([9], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        b = model.decode_fused(tok, pos)
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    for c0, c1 in zip(kc, model.k_cache):
+        assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
