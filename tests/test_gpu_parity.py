@@ -356,7 +356,13 @@ def test_decode_attention(heads, kv_heads, pos):
     qe, ke = rope(q), rope(k)
     kc0[0, :, pos] = ke
     vc0[0, :, pos] = v
-    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)  # cache rows written exactly as the reference would
+    # cache rows written as the reference would (cos/sin come from the device's cosf/sinf, so a
+    # rotated key may differ from torch's by an fp16 ulp); everything else untouched
+    assert torch.equal(vc, vc0)
+    assert torch.allclose(kc.float(), kc0.float(), atol=4e-3, rtol=2e-3)
+    untouched = torch.ones(max_len, dtype=torch.bool)
+    untouched[pos] = False
+    assert torch.equal(kc[0][:, untouched], kc0[0][:, untouched])
     rep = heads // kv_heads
     kk = kc0[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
     vv = vc0[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
