@@ -330,119 +330,183 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ out,
 }
 
 // ---------------------------------------------------------------------------
-// batched decompress -> LDS -> fp16 MFMA GEMM
+// batched decompress + fp16 MFMA GEMM
 // ---------------------------------------------------------------------------
-constexpr int kGemmThreads = 512;
+// out[b][row] = sum_col x[b][col] * W[row][col] with v_mfma_f32_16x16x32_f16:
+// M = 16 batch rows, N = the 16 lanes of a DPP row, K = 32 columns.
+//
+// The decode leaves, for every (tile row half mh, row half rh, kh), in lane
+// (g, a) the eight weights of matrix row 16*mh + 8*rh + a/2 at columns
+// 32*g' + 16*kh + 4*(a%2) + {0..3, 8..11} (g' = the lane group's tile block):
+// exactly the shape of an MFMA B operand (N index = a, K group = g), except
+// that even and odd lanes hold different columns (the 4*(a%2) term).  Each
+// product is therefore issued twice, once with the activations of columns
+// +0..3 / +8..11 and once with +4..7 / +12..15, into two accumulators; in the
+// first the even lanes' results are meaningful, in the second the odd lanes',
+// and the other half is simply never read.  That spends half of the matrix
+// core's work, which is free here (the kernel is bound by the decode), and
+// needs no data movement between decode and MFMA: the table lookups land in
+// the operand registers.
+constexpr int kGemmThreads = 512;  // 8 waves: up to 256 VGPRs for the accumulators
 constexpr int kGemmWaves = kGemmThreads / 64;
-constexpr int kStageStride = 128 + 8;                  // halfs per staged row (padding vs banks)
-constexpr int kStageHalfs = 32 * kStageStride;         // one wave's 32 x 128 tile
-constexpr int kStageBytes = kStageHalfs * 2;           // 8704
 
-// out[b][row] for b < batch.  NB = number of 16-wide batch tiles per pass.
-template <int K, int NB>
+// index into W[32] (lookup order of matvec_accumulate) of state (R, t, j)
+template <int K>
+__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
+  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
+  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
+}
+
+template <int K, int NB, int DEPTH>
 __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
     float* __restrict__ out, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
     const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16) {
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-  uint8_t* stage_all = smem + kLutBytes;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* red = reinterpret_cast<float*>(smem + kLut128Bytes);  // [kGemmWaves][32][16*NB]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int a = lane & 15, g = lane >> 4;
-  const uint32_t slot4 = (uint32_t)a << 2;
+  const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
   const int nkb = k >> 5;
-  const int nwl = (nkb + 3) >> 2;
-  const size_t rb_bytes = (size_t)nkb * 128 * K;
+  const int nwl = (nkb + 3) >> 2;  // wave-loads per row block; a partial last one reads zeros for x
   const int nrb = m >> 5;
-  constexpr int WL_BYTES = 512 * K;
-  uint16_t* stage = reinterpret_cast<uint16_t*>(stage_all + wave * kStageBytes);
-  float* red = reinterpret_cast<float*>(stage_all);  // reused after the k loop
+  const uint32_t rb_bytes = (uint32_t)nkb * 128 * K;
+  constexpr uint32_t WL_BYTES = 512 * K;
+  const uint32_t loff = (uint32_t)lane * 8 * K;
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
+  constexpr int NC = 16 * NB;
 
-  build_lut(lut, tlut, tid, kGemmThreads);
+  // items of this wave: (row block, wave-load wave + 8*j), flat, DEPTH in flight
+  const int npw = (nwl + kGemmWaves - 1) / kGemmWaves;
+  const int nvj = wave < nwl ? (nwl - wave + kGemmWaves - 1) / kGemmWaves : 0;
+  const int upw = (nrb - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int T = upw * npw;
+  int l_j = 0, l_t = 0;
+  uint32_t l_rboff = blockIdx.x * rb_bytes;
+  const uint32_t rb_step_bytes = gridDim.x * rb_bytes;
+  LaneData<K> buf[DEPTH];
+  auto issue = [&](int d) {
+    const bool valid = l_j < nvj && l_t < T;
+    const uint32_t wl = (uint32_t)(wave + l_j * kGemmWaves);
+    buf[d] = load_lane_buf<K>(rs_w, loff, valid ? l_rboff + wl * WL_BYTES : 0u);
+    ++l_t;
+    if (++l_j == npw) {
+      l_j = 0;
+      l_rboff += rb_step_bytes;
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue(d);
+  build_lut128(lut, tlut, tid, kGemmThreads);
   __syncthreads();
 
-  const int row16 = lane & 15, kgrp = lane >> 4;  // MFMA operand coordinates
+  // activations: lane (batch row a of tile nb, K group g) reads x[b][128*wl + 32*g + 16*kh + 0..15]
+  const uint16_t* xrow[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int bb = 16 * nb + a;
+    xrow[nb] = x + (size_t)(bb < batch ? bb : 0) * k + 32 * g;
+  }
 
-  for (int rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-    const uint8_t* base = packed + (size_t)rb * rb_bytes + (size_t)g * 128 * K + a * 8 * K;
-    float4_t acc[2][NB];
+  float4_t acc[2][2][2][NB];  // [mh][rh][column half][batch tile]
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[mt][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < 8 * NB; ++i) (&acc[0][0][0][0])[i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int wl = wave; wl < nwl; wl += kGemmWaves) {
-      const int kb = 4 * wl + g;
-      const bool active = kb < nkb;
-      uint32_t st[2][4][4];
-      if (active) {
-        const LaneData<K> ld = load_lane<K>(base + (size_t)wl * WL_BYTES);
-        lane_states<K>(ld, st);
-      }
+  int c_j = 0, c_rb = blockIdx.x;
+  for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int kh = t >> 1, mh = t & 1;
+    for (int d = 0; d < DEPTH; ++d) {
+      if (t + d < T && c_j < nvj) {
+        const int wl = wave + c_j * kGemmWaves;
+        // activations first (their latency hides behind the decode)
+        u32x4 xa[2][NB][2];  // [kh][nb][low / high 16 bytes]
+        const bool in_k = 128 * wl + 32 * g < k;  // false only in the lanes of a ragged last wave-load
+        const size_t xo = in_k ? (size_t)wl * 128 : 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int jh = j >> 1, rh = j & 1;
-          u32x2 v = {0u, 0u};
-          if (active) {
-            v[0] = lut_lookup(lut, st[0][t][j], slot4);
-            v[1] = lut_lookup(lut, st[1][t][j], slot4);
+        for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const u32x4* px = reinterpret_cast<const u32x4*>(xrow[nb] + xo + 16 * kh);
+            xa[kh][nb][0] = px[0];
+            xa[kh][nb][1] = px[1];
           }
-          const int row = 16 * mh + 8 * rh + (a >> 1);
-          const int col = 32 * g + 16 * kh + 8 * jh + 4 * (a & 1);
-          *reinterpret_cast<u32x2*>(stage + row * kStageStride + col) = v;
+        if (!in_k) {
+          // columns past k: zero activations cancel whatever the lane decodes
+#pragma unroll
+          for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              xa[kh][nb][0] = u32x4{0u, 0u, 0u, 0u};
+              xa[kh][nb][1] = u32x4{0u, 0u, 0u, 0u};
+            }
         }
+        uint32_t P[16], W[32];
+        packed_states<K>(buf[d], P);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
+          W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
+          W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+          for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+              const int tt = 2 * kh + mh;
+              const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
+                                W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
+              const half8_t bop = __builtin_bit_cast(half8_t, wv);
+#pragma unroll
+              for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int ch = 0; ch < 2; ++ch) {
+                  // columns +4*ch+{0..3} and +8+4*ch+{0..3} of the 16 loaded ones
+                  const u32x4 xv = {xa[kh][nb][0][2 * ch], xa[kh][nb][0][2 * ch + 1],
+                                    xa[kh][nb][1][2 * ch], xa[kh][nb][1][2 * ch + 1]};
+                  acc[mh][rh][ch][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                      __builtin_bit_cast(half8_t, xv), bop, acc[mh][rh][ch][nb], 0, 0, 0);
+                }
+            }
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const size_t kcol0 = (size_t)wl * 128;
+      issue(d);
+      if (t + d < T && ++c_j == npw) {
+        // ---- end of a row block: pick the meaningful accumulator, add the
+        // partner lane, reduce across waves, store
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int kc = 32 * ks + 8 * kgrp;
-        half8_t bfrag[NB];
+        for (int mh = 0; mh < 2; ++mh)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const int b = 16 * nb + row16;
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (b < batch && kcol0 + kc < (size_t)k)
-            raw = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + kcol0 + kc);
-          bfrag[nb] = __builtin_bit_cast(half8_t, raw);
+          for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                float v = (a & 1) ? acc[mh][rh][1][nb][i] : acc[mh][rh][0][nb][i];
+                v += dpp_xor1(v);
+                acc[mh][rh][0][nb][i] = 0.f;
+                acc[mh][rh][1][nb][i] = 0.f;
+                // lane (g, a even): batch row 16*nb + 4*g + i, matrix row 16*mh + 8*rh + a/2
+                if ((a & 1) == 0)
+                  red[(wave * 32 + 16 * mh + 8 * rh + (a >> 1)) * NC + 16 * nb + 4 * g + i] = v;
+              }
+        __syncthreads();
+        for (int e = tid; e < 32 * NC; e += kGemmThreads) {
+          const int bb = e >> 5, row = e & 31;  // consecutive threads -> consecutive rows of out
+          float sum = 0.f;
+#pragma unroll
+          for (int w = 0; w < kGemmWaves; ++w) sum += red[(w * 32 + row) * NC + bb];
+          if (round_f16) sum = (float)(_Float16)sum;
+          if (bb < batch) out[(size_t)bb * m + c_rb * 32 + row] = sum;
         }
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const half8_t afrag = *reinterpret_cast<const half8_t*>(
-              stage + (16 * mt + row16) * kStageStride + kc);
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-            acc[mt][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag[nb], acc[mt][nb], 0, 0, 0);
-        }
+        __syncthreads();
+        c_j = 0;
+        c_rb += gridDim.x;
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
     }
-
-    // cross-wave reduction: red[wave][row 32][col 16*NB]
-    __syncthreads();
-    constexpr int NC = 16 * NB;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          red[(wave * 32 + 16 * mt + 4 * kgrp + i) * NC + 16 * nb + row16] = acc[mt][nb][i];
-    __syncthreads();
-    for (int e = tid; e < 32 * NC; e += kGemmThreads) {
-      const int b = e >> 5, row = e & 31;  // consecutive threads -> consecutive rows of out
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < kGemmWaves; ++w) sum += red[(w * 32 + row) * NC + b];
-      if (round_f16) sum = (float)(_Float16)sum;
-      if (b < batch) out[(size_t)b * m + rb * 32 + row] = sum;
-    }
-    __syncthreads();
   }
 }
 
@@ -477,7 +541,7 @@ hipError_t allow_lds(F* fn, size_t bytes) {
                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-constexpr size_t kGemmLds = kLutBytes + kGemmWaves * kStageBytes;
+constexpr size_t kGemmLds = kLut128Bytes + (size_t)kGemmWaves * 32 * 32 * sizeof(float);
 
 hipError_t setup_once() {
   static hipError_t status = [] {
@@ -493,15 +557,12 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((gemm_kernel<2, 1>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<2, 2>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<2, 4>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 1>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 2>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 4>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 1>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 2>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 4>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 1, 4>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 2, 4>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 1, 3>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 2, 3>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 1, 2>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 2, 2>), kGemmLds)
 #undef QTIP_ALLOW
     return hipSuccess;
   }();
@@ -681,17 +742,16 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   hipStream_t st = (hipStream_t)stream;
   auto* p = (const uint8_t*)packed;
   auto* t = (const uint32_t*)tlut;
-  // batch handled in passes of at most 64 rows
-  for (int b0 = 0; b0 < batch; b0 += 64) {
-    const int nb = batch - b0 < 64 ? batch - b0 : 64;
+  // batch handled in passes of at most 32 rows (two 16-row MFMA tiles)
+  for (int b0 = 0; b0 < batch; b0 += 32) {
+    const int nb = batch - b0 < 32 ? batch - b0 : 32;
     float* o = out + (size_t)b0 * m;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
 #define QTIP_GEMM(KB, NBT) \
-  gemm_kernel<KB, NBT><<<grid, kGemmThreads, kGemmLds, st>>>(o, p, xx, t, m, k, nb, round_f16)
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2)><<<grid, kGemmThreads, kGemmLds, st>>>(o, p, xx, t, m, k, nb, round_f16)
 #define QTIP_GEMM_K(KB)            \
   if (nb <= 16) QTIP_GEMM(KB, 1);  \
-  else if (nb <= 32) QTIP_GEMM(KB, 2); \
-  else QTIP_GEMM(KB, 4);
+  else QTIP_GEMM(KB, 2);
     switch (bits) {
       case 2: QTIP_GEMM_K(2) break;
       case 3: QTIP_GEMM_K(3) break;
