@@ -40,6 +40,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--workload", choices=["70b", "7b"], default="70b")
+    ap.add_argument("--shape", default=None,
+                    help="restrict the set to one of its matrices (qkv, o, up_gate, down): used for per-kernel "
+                         "counter runs under rocprofv3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer timings")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -61,6 +64,10 @@ def main():
     torch.cuda.set_device(dev)
     K = args.bits
     shapes = SHAPES_70B if args.workload == "70b" else SHAPES_7B
+    if args.shape is not None:
+        shapes = [sh for sh in shapes if sh[0] == args.shape]
+        if not shapes:
+            ap.error(f"unknown --shape {args.shape}")
     set_bytes = sum(m * k * K // 8 for _, m, k in shapes)
     copies = max(2, -(-(600 << 20) // set_bytes))
 
@@ -155,7 +162,7 @@ def main():
             "avg_launch_us": round(avg_launch_us, 3),
             "bytes_per_launch": set_bytes // len(shapes),
             "traffic": (round(MEASURED_TRAFFIC_RATIO[(args.workload, K)] * set_bytes / len(shapes))
-                        if (args.workload, K) in MEASURED_TRAFFIC_RATIO else None),
+                        if (args.workload, K) in MEASURED_TRAFFIC_RATIO and args.shape is None else None),
             "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, see profiles/)",
         },
         "host_wall_s_timed_region": round(wall_s, 4),

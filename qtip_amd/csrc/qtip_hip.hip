@@ -303,6 +303,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
           acc[i] = 0.f;
         }
+#if !defined(QTIP_ABLATE_FLUSH)
         __syncthreads();
         if (tid < 32) {
           float sum = 0.f;
@@ -310,6 +311,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           for (int w = 0; w < kWaves; ++w) sum += pp[w * 32 + tid];
           out_s[c_rb * 32 + tid] = sum;
         }
+#endif
         parity ^= 1;  // the other buffer is free: its readers passed the barrier above
         c_j = 0;
         c_rb += rb_step;
