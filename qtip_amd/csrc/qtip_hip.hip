@@ -20,19 +20,6 @@ __device__ __forceinline__ float dpp_xor1(float v) {
       float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1 /* quad_perm 1,0,3,2 */,
                                          0xF, 0xF, false));
 }
-__device__ __forceinline__ float swz_xor16(float v) {
-  return __builtin_bit_cast(float,
-                            __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
-}
-__device__ __forceinline__ float xor32(float v) {
-  uint32_t u = __builtin_bit_cast(uint32_t, v);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  // r[0]: lanes 0-31 keep their value, lanes 32-63 receive lanes 0-31;
-  // r[1]: lanes 0-31 receive lanes 32-63, lanes 32-63 keep theirs.
-  const bool upper = (threadIdx.x & 32) != 0;
-  return __builtin_bit_cast(float, upper ? r[0] : r[1]);
-}
-
 // ---------------------------------------------------------------------------
 // decode: packed stream -> dense fp16 (m, k)
 // ---------------------------------------------------------------------------
@@ -81,43 +68,55 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // decompress + matvec
 // ---------------------------------------------------------------------------
 constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
+#ifndef QTIP_D2X
+#define QTIP_D2X 6
+#endif
+constexpr int kD2X = QTIP_D2X;
 constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a workgroup's k range
 
-// 32 states of one wave-load.  All hashes, addresses and the 32 table reads
-// are issued first and the 32 dot products follow, so a read has the rest of
-// the address arithmetic (a few hundred cycles) to come back from LDS.
-// slot4 = LDS address of the table + 4 * (lane % 32);
-// acc[2*mh + rh] belongs to row 16*mh + 8*rh + a/2 of the 32-row block.
+// index into W[32] (lookup order of matvec_accumulate) of state (R, t, j)
+template <int K>
+__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
+  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
+  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
+}
+
+// 32 states of one wave-load.  All hashes, addresses and the 32 table reads are issued first, so
+// a read has the rest of the address arithmetic (a few hundred cycles) to come back from LDS;
+// the products run on the matrix core, which leaves the vector ALU to the decode (a v_dot2c per
+// state measured 5 % slower end to end).  The four table words of a
+// (tile row half mh, row half rh, kh) group are a v_mfma_f32_16x16x32_f16 B operand (N = the 16
+// lanes `a` of a DPP row, K group = g), the lane's own eight x values of that kh are the A operand
+// row `a`: D[i][j] = sum over (g, 8 halves) of x(lane i) * W(lane j), which is the wanted dot
+// product whenever lanes i and j read the same columns, i.e. i % 2 == j % 2.  Lane (g, a) keeps
+// D[4g + r][a] in element r, so element a % 2 of the accumulator is the lane's row sum over all
+// four blocks of the wave-load (the cross-block reduction happens inside the MFMA).
 template <int K>
 __device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u32x2 xv[4],
-                                                  uint32_t slot4, float acc[4]) {
+                                                       uint32_t slot4, float4_t acc[4]) {
   uint32_t P[16], W[32];
   packed_states<K>(ld, P);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
-#if defined(QTIP_ABLATE_LDS)
-    W[2 * i] = lut128_addr_lo(q, slot4);
-    W[2 * i + 1] = lut128_addr_hi(q, slot4);
-#else
     W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
     W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
-#endif
   }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int R = PkMeta<K>::R(i);
+  for (int kh = 0; kh < 2; ++kh) {
+    const u32x4 xa = {xv[2 * kh][0], xv[2 * kh][1], xv[2 * kh + 1][0], xv[2 * kh + 1][1]};
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      // (copy the vector element to a scalar first: bit_cast applied directly
-      // to a vector-element lvalue reads element 0)
-      const uint32_t xr = xv[PkMeta<K>::xq(i, hh)][R];
-      acc[PkMeta<K>::acc(i, hh)] =
-          __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, W[2 * i + hh]),
-                                 __builtin_bit_cast(half2_t, xr), acc[PkMeta<K>::acc(i, hh)], false);
-    }
+    for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh) {
+        const int tt = 2 * kh + mh;
+        const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
+                          W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
+        acc[2 * mh + rh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            __builtin_bit_cast(half8_t, xa), __builtin_bit_cast(half8_t, wv), acc[2 * mh + rh], 0, 0, 0);
+      }
   }
 }
 
@@ -127,7 +126,10 @@ template <int K>
 __device__ __forceinline__ LaneData<K> load_lane_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
                                                      uint32_t soff) {
   LaneData<K> r;
-  constexpr int NT = 2;  // non-temporal: the stream is read once
+#ifndef QTIP_NT
+#define QTIP_NT 2
+#endif
+  constexpr int NT = QTIP_NT;  // non-temporal: the stream is read once
   if constexpr (K == 2) {
     const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
 #pragma unroll
@@ -158,16 +160,10 @@ __device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t
   for (int q = 0; q < 4; ++q) xv[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff + 16 * q, soff, 0);
 }
 
-__device__ __forceinline__ void load_x(const uint16_t* __restrict__ xw, uint32_t xoff, u32x2 xv[4]) {
-  const uint8_t* p = reinterpret_cast<const uint8_t*>(xw) + xoff;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) xv[q] = *reinterpret_cast<const u32x2*>(p + 16 * q);
-}
-
 // Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup take
 // the unit's wave-loads round-robin (so the workgroup streams one contiguous
-// run of bytes), reduce across lanes with DPP / ds_swizzle / permlane swaps and
-// across waves through LDS in a fixed order, and store 32 sums to
+// run of bytes), reduce across the four blocks of a wave-load inside the MFMA, across the two
+// column halves with one DPP exchange and across waves through LDS in a fixed order, and store 32 sums to
 // dst[s*m + 32*rb ...]: the result itself when S == 1, else one of S partial
 // vectors that the consumer adds in order (deterministic either way).
 //
@@ -240,26 +236,51 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       l_rboff += rb_step_bytes;
     }
   };
-  // the first loads go out before the table is built
+  // Prologue loads in the order they are needed: the table words and x first, then the first
+  // DEPTH wave-loads of the stream.  Loads return in order, so the table build only waits for its
+  // own few words while the (much larger) stream requests are still on their way.
+  static_assert(kLutEntries * 8 == 8 * kThreads, "table build assumes 8 16-byte items per thread");
+  uint32_t tw[4];  // item it*1024 + tid belongs to entry it*128 + tid/8; entries e and e+512 share a word
+#pragma unroll
+  for (int it = 0; it < 4; ++it) tw[it] = tlut[it * 128 + (tid >> 3)];
+  u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+  if constexpr (XLDS) {
+    // x of wave-loads [wl0, wl1): 16 bytes per thread and pass, at most 2 passes (28 KiB)
+    const int xbytes = (wl1 - wl0) * 256;
+    const int kbytes = k * 2;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+      const int o = (ps * kThreads + tid) * 16;
+      if (o < xbytes && wl0 * 256 + o < kbytes)
+        xstage[ps] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(x) + (size_t)wl0 * 256 + o);
+    }
+  }
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(d);
 
-  build_lut128(lut, tlut, tid, kThreads);
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const uint32_t w = tw[it & 3] ^ ((uint32_t)(it >> 2) << 15);
+    const u32x4 v = {w, w, w, w};
+    reinterpret_cast<u32x4*>(lut)[it * kThreads + tid] = v;
+  }
   if constexpr (XLDS) {
-    // x of wave-loads [wl0, wl1): 16 bytes per thread and pass
     const int xbytes = (wl1 - wl0) * 256;
-    const int kbytes = k * 2;
-    for (int o = tid * 16; o < xbytes; o += kThreads * 16) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (wl0 * 256 + o < kbytes)
-        v = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(x) + (size_t)wl0 * 256 + o);
-      *reinterpret_cast<u32x4*>(xs_lds + o) = v;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+      const int o = (ps * kThreads + tid) * 16;
+      if (o < xbytes) *reinterpret_cast<u32x4*>(xs_lds + o) = xstage[ps];
     }
   }
   __syncthreads();
   const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)wave * 256u;  // wave-load w_first
 
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[4];  // [2*mh + rh]: rows 16*mh + 8*rh + a/2 of the unit's 32-row block
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+  auto accumulate = [&](const LaneData<K>& ld, const u32x2 xv[4]) {
+    matvec_accumulate<K>(ld, xv, slot4, acc);
+  };
   int parity = 0, c_j = 0, c_rb = rb0;
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
@@ -272,9 +293,9 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
             const uint32_t xa = xs_lane + (uint32_t)c_j * (kWaves * 256u);
 #pragma unroll
             for (int q = 0; q < 4; ++q) xv[q] = *(lds_u32x2_t*)(uintptr_t)(xa + 16u * q);
-            matvec_accumulate<K>(buf[d], xv, slot4, acc);
+            accumulate(buf[d], xv);
           } else {
-            matvec_accumulate<K>(buf[d], xbuf[d], slot4, acc);
+            accumulate(buf[d], xbuf[d]);
           }
         }
       }
@@ -283,27 +304,25 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       issue(d);
       if (t + d < T && ++c_j == npw) {
         // ---- end of a unit: ragged tail, reductions, store
-        // k/32 not a multiple of 4: one wave takes the partial wave-load with
-        // the lanes of the missing blocks switched off
-        if (tail_wave && 4 * nfull + g < nkb) {
+        // k/32 not a multiple of 4: one wave takes the partial wave-load.  Every lane takes part
+        // in an MFMA, so the lanes of the missing blocks read x = 0 (the descriptor of x ends
+        // at k) and whatever follows in the stream (0 past its end).
+        if (tail_wave) {
           u32x2 xt[4];
-          load_x(x + (size_t)nfull * 128, xoff, xt);
+          load_x_buf(rs_x, xoff, (uint32_t)nfull * 256u, xt);
           const LaneData<K> tail =
-              load_lane<K>(packed + (size_t)c_rb * rb_bytes + (size_t)nfull * WL_BYTES + loff);
-          matvec_accumulate<K>(tail, xt, slot4, acc);
+              load_lane_buf<K>(rs_w, loff, (uint32_t)c_rb * rb_bytes + (uint32_t)nfull * WL_BYTES);
+          accumulate(tail, xt);
         }
         float* pp = part + parity * (kWaves * 32);
-        // lanes sharing a row differ in lane bits 0 (column half), 4 and 5 (block)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float v = acc[i];
+          // element a % 2 holds the lane's sum over the four blocks; add the other column half
+          float v = (a & 1) ? acc[i][1] : acc[i][0];
           v += dpp_xor1(v);
-          v += swz_xor16(v);
-          v += xor32(v);
+          acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
           if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
-          acc[i] = 0.f;
         }
-#if !defined(QTIP_ABLATE_FLUSH)
         __syncthreads();
         if (tid < 32) {
           float sum = 0.f;
@@ -311,7 +330,6 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           for (int w = 0; w < kWaves; ++w) sum += pp[w * 32 + tid];
           out_s[c_rb * 32 + tid] = sum;
         }
-#endif
         parity ^= 1;  // the other buffer is free: its readers passed the barrier above
         c_j = 0;
         c_rb += rb_step;
@@ -351,13 +369,6 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ out,
 // the operand registers.
 constexpr int kGemmThreads = 512;  // 8 waves: up to 256 VGPRs for the accumulators
 constexpr int kGemmWaves = kGemmThreads / 64;
-
-// index into W[32] (lookup order of matvec_accumulate) of state (R, t, j)
-template <int K>
-__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
-  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
-  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
-}
 
 template <int K, int NB, int DEPTH>
 __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
@@ -556,7 +567,7 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 4, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<3, 3, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, kD2X, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4>), kGemmLds)
@@ -673,7 +684,7 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {
-      case 2: matvec_kernel<2, 6, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, kD2X, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
       case 3: matvec_kernel<3, 4, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
       default: matvec_kernel<4, 3, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
     }

@@ -101,15 +101,15 @@ def decompress_matvec(packed, x, tlut, m, k, bits, out=None, split_k=True):
     return out
 
 
-def decompress_matvec_parts(packed, x, tlut, m, k, bits):
+def decompress_matvec_parts(packed, x, tlut, m, k, bits, nparts=None):
     """(S, m) fp32 partial sums of decode(packed) @ x over S ranges of k; their
-    sum over axis 0 (in order) is the matvec.  S = matvec_split(...)."""
+    sum over axis 0 (in order) is the matvec.  S = nparts or matvec_split(...)."""
     _check_packed(packed, m, k, bits)
     _check_tlut(tlut, packed.device)
     require_cuda(x, "x", torch.float16)
     if x.numel() != k or x.device != packed.device:
         raise ValueError(f"x must hold {k} fp16 values on {packed.device}")
-    S = matvec_split(m, k, bits, packed.device)
+    S = int(nparts) if nparts is not None else matvec_split(m, k, bits, packed.device)
     parts = torch.empty((S, m), dtype=torch.float32, device=packed.device)
     with torch.cuda.device(packed.device):
         check(lib().qtip_decompress_matvec_parts(_ptr(parts), _ptr(packed), _ptr(x), _ptr(tlut), m, k, bits, S,
