@@ -143,6 +143,35 @@ int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
                           const void* pos_i64, const float* inv_freq, int heads, int kv_heads,
                           int head_dim, int max_len, void* stream);
 
+/* ---- packing tools (natural packing = one circular big-endian bitstream per tile, stored as
+ * T*K/16 little-endian uint16 words; state i is the 16-bit window at bit i*K*V) ---------------- */
+
+/* Byte permutation between the natural packing and the kernel packing of a 16x16-tile, V=2
+ * matrix, m*k*bits/8 bytes each way; out and in must not overlap.
+ * to_kernel != 0: natural -> kernel, the re-pack of lib/algo/finetune.py:196-201;
+ * to_kernel == 0: kernel -> natural, lib/utils/kernel_decompress.py:19-24. */
+int qtip_repack(void* out, const void* in, int m, int k, int bits, int to_kernel, void* stream);
+
+/* Natural packing -> explicit states, states[ntiles][T/V] (int32, values < 65536).
+ * Replaces bitshift_codebook.unpack_trellis (lib/codebook/bitshift.py:329-353).
+ * L = 16; T = weights per tile; needs T % V == 0, (T*K) % 16 == 0, V in {1,2}, K*V <= 16. */
+int qtip_unpack_trellis(int32_t* states, const void* packed, long ntiles, int T, int K, int V,
+                        void* stream);
+
+/* States -> natural packing (packed[ntiles][T*K/16] uint16).  Replaces
+ * bitshift_codebook.pack_trellis (lib/codebook/bitshift.py:294-327).  *violations (device int,
+ * zeroed by the caller) receives the number of consecutive state pairs that do not overlap by
+ * 16 - K*V bits; the reference asserts that there are none (:307-309). */
+int qtip_pack_trellis(void* packed, const int32_t* states, long ntiles, int T, int K, int V,
+                      int* violations, void* stream);
+
+/* Natural packing -> dense (m, n) matrix for any decode mode: lut is the expanded table
+ * [V][65536] (cb.lut of the reference, QTIP_F16 or QTIP_F32), out has the table's dtype.
+ * Replaces BitshiftLinear.get_hatW(cb.unpack_trellis(...)) (lib/codebook/bitshift.py:199-201,
+ * 329-353, 378-381), the path taken when has_kernel is false. */
+int qtip_decode_natural(void* out, const void* packed, const void* lut, int lut_dtype, int m, int n,
+                        int td_x, int td_y, int K, int V, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,14 @@ Pinning status of each function (what, other than itself, fixes its result):
                           "parity unpinned" and checked by tolerance only.
   bitshift_linear_forward dense W_eff formula of lib/codebook/bitshift.py:389-413
                           (the reference's own "manifest" form).
+  unpack_trellis_generic  any (T, K, V): equal to unpack_trellis_natural for the 16x16,
+  pack_trellis_generic    V=2 case; round trip; bit-level definition by Python-int
+  decode_natural_generic  string slicing in the tests; the 16x16/V=2 case equals decode_natural.
+  code_1mad / code_2mad   byte-sum codes: scalar Python-int recomputation, exact moments
+                          (mean 0, variance 1 over all 2^32 inputs follows from the byte-sum
+                          construction; sqrt(21845) = 147.8005...), value grid k/147.8.
+  code_3inst              scalar Python-int + struct('e') recomputation of hand-picked states.
+  quantlut                closed form; equals quantlut_sym up to the sign of element 0.
 """
 from __future__ import annotations
 
@@ -385,3 +393,91 @@ def dense_equivalent(packed, SU, SV, tlut, K):
     a = hadamard_transform(w, transpose=False)  # (HL @ w^T)^T, shape (m, n)
     b = hadamard_transform(a.T, transpose=False).T  # HR applied over the m axis
     return (SV[:, None] * 32.0) * b * SU[None, :]
+
+
+# ----------------------------------------------------------------------------
+# f3. generic natural packing (any tile size T, K bits, V weights per state) and
+#     the other decode modes of the codebook
+# ----------------------------------------------------------------------------
+
+
+def unpack_trellis_generic(words: np.ndarray, T: int, K: int, V: int) -> np.ndarray:
+    """(ntiles, T*K/16) uint16 -> (ntiles, T/V) int32 states, lib/codebook/bitshift.py:329-353
+    for any tile size: circular stream of T*K bits, state i = 16-bit window at bit i*K*V."""
+    nw = T * K // 16
+    words = np.ascontiguousarray(words).view(np.uint16).reshape(-1, nw)
+    nt = words.shape[0]
+    bits = ((words[:, :, None] >> (15 - np.arange(16, dtype=np.uint16))) & 1).reshape(nt, T * K).astype(np.int64)
+    kv = K * V
+    ext = np.concatenate([bits, bits[:, :L_BITS - kv]], axis=1) if kv < L_BITS else bits
+    weights = 1 << np.arange(15, -1, -1, dtype=np.int64)
+    ns = T // V
+    states = np.empty((nt, ns), dtype=np.int32)
+    for i in range(ns):
+        states[:, i] = (ext[:, i * kv:i * kv + 16] * weights).sum(axis=1)
+    return states
+
+
+def pack_trellis_generic(states: np.ndarray, K: int, V: int) -> np.ndarray:
+    """(ntiles, T/V) states -> (ntiles, T*K/16) uint16, lib/codebook/bitshift.py:294-327: all 16
+    bits of state 0, then the K*V fresh bits of every later state, cut to T*K bits."""
+    states = np.asarray(states, dtype=np.int64)
+    nt, ns = states.shape
+    kv = K * V
+    low = (1 << (L_BITS - kv)) - 1
+    if not np.all((states[:, :-1] & low) == (states[:, 1:] >> kv)):
+        raise ValueError("states are not a bitshift trellis walk")
+    bits = np.zeros((nt, ns * kv + L_BITS - kv), dtype=np.uint8)
+    bits[:, :16] = (states[:, :1] >> np.arange(15, -1, -1)) & 1
+    for i in range(1, ns):
+        fresh = states[:, i] & ((1 << kv) - 1)
+        bits[:, 16 + (i - 1) * kv:16 + i * kv] = (fresh[:, None] >> np.arange(kv - 1, -1, -1)) & 1
+    bits = bits[:, :ns * kv]
+    w = bits.reshape(nt, -1, 16).astype(np.uint32)
+    return (w << np.arange(15, -1, -1, dtype=np.uint32)).sum(axis=2).astype(np.uint16)
+
+
+def decode_natural_generic(words, lut, m, n, td_x, td_y, K, V):
+    """Natural stream -> (m, n) in lut's dtype; lut is (V, 65536).  lib/codebook/bitshift.py:199-201
+    (recons) and :378-381 (get_hatW): sequence position i*V + v of a tile is its row-major element."""
+    st = unpack_trellis_generic(words, td_x * td_y, K, V)  # (ntiles, T/V)
+    seq = np.stack([lut[v][st] for v in range(V)], axis=-1).reshape(-1, td_x * td_y)
+    return np.ascontiguousarray(
+        seq.reshape(m // td_x, n // td_y, td_x, td_y).transpose(0, 2, 1, 3).reshape(m, n))
+
+
+def _byte_sum(x):
+    return ((x & 255) + ((x >> 8) & 255) + ((x >> 16) & 255) + ((x >> 24) & 255)).astype(np.int64)
+
+
+def code_1mad(states: np.ndarray) -> np.ndarray:
+    """lib/codebook/bitshift.py:17-26, uint64 arithmetic reduced mod 2^32."""
+    x = (np.asarray(states, dtype=np.uint64) * np.uint64(34038481) + np.uint64(76625530)) & np.uint64(0xFFFFFFFF)
+    return ((_byte_sum(x) - 510).astype(np.float32) / np.float32(147.800537109375)).astype(np.float32)
+
+
+def code_2mad(states: np.ndarray) -> np.ndarray:
+    """lib/codebook/bitshift.py:29-40."""
+    M = np.uint64(0xFFFFFFFF)
+    x = (np.asarray(states, dtype=np.uint64) * np.uint64(264435761) + np.uint64(1013904223)) & M
+    x = (((x * np.uint64(1664525)) >> np.uint64(32)) + x) & M
+    return ((_byte_sum(x) - 510).astype(np.float32) / np.float32(147.800537109375)).astype(np.float32)
+
+
+def code_3inst(states: np.ndarray) -> np.ndarray:
+    """lib/codebook/bitshift.py:43-59: the two 16-bit halves of ((x*a+b) & 0x8FFF8FFF) ^ 0x3B603B60
+    read as fp16 and added in fp16."""
+    M = np.uint64(0xFFFFFFFF)
+    x = (np.asarray(states, dtype=np.uint64) * np.uint64(89226354) + np.uint64(64248484)) & M
+    res = (x & np.uint64(0x8FFF8FFF)) ^ np.uint64(996162400)
+    top = (res >> np.uint64(16)).astype(np.uint16).view(np.float16)
+    bot = (res & np.uint64(0xFFFF)).astype(np.uint16).view(np.float16)
+    return (top + bot).astype(np.float32)
+
+
+def quantlut(tlut: np.ndarray) -> np.ndarray:
+    """lib/codebook/bitshift.py:62-69: tlut[(s*(s+1) >> (16-nbits)) & (2^nbits - 1)] for all states."""
+    nbits = int(np.log2(tlut.shape[0]))
+    s = np.arange(1 << L_BITS, dtype=np.int64)
+    idx = ((s * (s + 1)) >> (16 - nbits)) & ((1 << nbits) - 1)
+    return tlut[idx]

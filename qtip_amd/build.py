@@ -4,7 +4,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRCS = [os.path.join(HERE, "csrc", f) for f in ("qtip_hip.hip", "qtip_rht.hip", "qtip_decoder.hip")]
+SRCS = [os.path.join(HERE, "csrc", f) for f in ("qtip_hip.hip", "qtip_rht.hip", "qtip_decoder.hip", "qtip_pack.hip")]
 OUT = os.path.join(HERE, "libqtip_hip.so")
 
 # packed fp32 VALU forms are switched off for every HIP translation unit

@@ -4,7 +4,9 @@ Kept from the reference: class names, constructor and forward signatures,
 attribute names (`cb`, `scale`, `internal_dtype`, `has_kernel`), tensor
 layouts and the cast points of the forward pass.  The quantiser side of
 `bitshift_codebook` (Viterbi, `quantize`, `update`) is not part of the
-inference path and raises NotImplementedError.
+inference path and raises NotImplementedError.  Every decode mode of the
+reference is available on the natural-packing path; the fused kernels cover
+the HYB code ('quantlut_sym', has_kernel).
 """
 import math
 
@@ -30,9 +32,56 @@ def quantlut_sym(tlut, L, nbits):
     return lut
 
 
+def _byte_sum_code(x):
+    """Sum of the four bytes of a 32-bit word, centred and scaled to unit variance: the value map
+    shared by the computed codes '1mad' and '2mad' (lib/codebook/bitshift.py:17-40)."""
+    y = sum((x >> sh) & 255 for sh in (0, 8, 16, 24)) - 510
+    return y.to(torch.float32) / 147.800537109375
+
+
+def decode_1mad(x):
+    """'1mad' computed code (lib/codebook/bitshift.py:17-26): one 32-bit multiply-add, byte sum."""
+    m32 = (1 << 32) - 1
+    x = ((x.to(torch.int64) & m32) * 34038481 + 76625530) & m32
+    return _byte_sum_code(x)
+
+
+def decode_2mad(x):
+    """'2mad' computed code (lib/codebook/bitshift.py:29-40): LCG step, multiply-high add, byte sum."""
+    m32 = (1 << 32) - 1
+    x = ((x.to(torch.int64) & m32) * 264435761 + 1013904223) & m32
+    x = (((x * 1664525) >> 32) + x) & m32
+    return _byte_sum_code(x)
+
+
+def decode_3inst(x):
+    """'3inst' computed code (lib/codebook/bitshift.py:43-59): multiply-add, keep sign and 12
+    mantissa/exponent bits of each half, xor a constant exponent pattern in, add the two fp16s."""
+    m32 = (1 << 32) - 1
+    x = ((x.to(torch.int64) & m32) * 89226354 + 64248484) & m32
+    keep = (1 << 15) + ((1 << 12) - 1)
+    res = (x & ((keep << 16) + keep)) ^ 996162400
+    halves = torch.stack([res >> 16, res & 0xFFFF]).to(torch.int32)
+    fp = (halves - ((halves >= 1 << 15).to(torch.int32) << 16)).to(torch.int16).view(torch.float16)
+    return (fp[0] + fp[1]).float()
+
+
+def quantlut(tlut, L, nbits):
+    """Expansion of a tunable table without the sign trick (lib/codebook/bitshift.py:62-69)."""
+    with torch.no_grad():
+        s = torch.arange(1 << L, device=tlut.device)
+        idx = (((s + 1) * s) >> (16 - nbits)) & ((1 << nbits) - 1)
+    return tlut[idx]
+
+
+_COMPUTED = {'1mad': decode_1mad, '2mad': decode_2mad, '3inst': decode_3inst}
+
+
 class bitshift_codebook(nn.Module):
-    """Inference part of the reference class (lib/codebook/bitshift.py:83-201):
-    holds the tunable table and its expansion; `recons` maps states to weights."""
+    """Decode side of the reference class (lib/codebook/bitshift.py:83-201, 294-353): holds the
+    expanded table `lut` (V, 2**L) of the chosen decode mode ('lut', '1mad', '2mad', '3inst',
+    'quantlut', 'quantlut_sym'), maps states to weights (`recons`) and converts between states and
+    the natural packing.  The quantiser side (Viterbi search) raises NotImplementedError."""
 
     def __init__(self, L=16, K=2, V=2, tlut_bits=16, decode_mode='lut', tlut=None):
         super().__init__()
@@ -41,33 +90,66 @@ class bitshift_codebook(nn.Module):
         self.L, self.K, self.V = L, K, V
         self.tlut_bits = tlut_bits
         self.decode_mode = decode_mode
-        if decode_mode != 'quantlut_sym':
-            raise NotImplementedError(f"decode_mode {decode_mode!r}: only the HYB code 'quantlut_sym' is built")
-        if V != 2:
-            raise NotImplementedError("quantlut_sym needs V == 2")
-        if tlut is None:
-            # the reference fits a k-means table here (bitshift.py:147-168); a
-            # checkpoint always overwrites it, so start from a seeded Gaussian table
-            g = torch.Generator().manual_seed(0)
-            tlut = torch.randn(2**tlut_bits, V, generator=g)
-            tlut = (tlut / tlut.std(unbiased=False)) * 0.9682458365518543
-            self.register_buffer('tlut', tlut)
-            self.register_buffer('lut', quantlut_sym(self.tlut, L, tlut_bits).T.contiguous())
+        if L != 16:
+            raise NotImplementedError("only L = 16 trellises are built (16-bit state windows)")
+        if decode_mode in _COMPUTED:
+            if V != 1:
+                raise ValueError(f"decode_mode {decode_mode!r} needs V == 1")
+            self.register_buffer('lut', _COMPUTED[decode_mode](torch.arange(2**L)).unsqueeze(0))
+        elif decode_mode in ('lut', 'quantlut', 'quantlut_sym'):
+            if tlut is None:
+                self.register_buffer('tlut', self._default_tlut())
+                self.register_buffer('lut', self._expand().T.contiguous())
+            else:
+                self.tlut = tlut
+                self.recons_lut()
         else:
-            self.tlut = tlut
-            self.recons_lut()
+            raise ValueError(f"unknown decode_mode {decode_mode!r}")
         self.version = 0
 
+    def _default_tlut(self):
+        """Start tables of lib/codebook/bitshift.py:106-168 (a checkpoint overwrites them)."""
+        n, V = 2**self.tlut_bits, self.V
+        if self.decode_mode == 'lut':
+            if self.tlut_bits != self.L:
+                raise ValueError("decode_mode 'lut' needs tlut_bits == L")
+            return torch.randn(n, V)
+        if self.decode_mode == 'quantlut':
+            if V == 1:
+                return (torch.erfinv((torch.arange(n) + 0.5) / n * 2 - 1) * 2.0**0.5).unsqueeze(-1)
+            if V == 2:
+                R = ((n / (n - torch.arange(n))).log() * 2).sqrt()
+                return torch.stack([R * torch.arange(n).sin(), R * torch.arange(n).cos()], dim=-1)
+            raise ValueError("quantlut needs V in {1, 2}")
+        if V != 2:
+            raise ValueError("quantlut_sym needs V == 2")
+        # the reference fits a k-means table to Gaussian samples here; start from a seeded
+        # Gaussian table with the same normalisation instead
+        g = torch.Generator().manual_seed(0)
+        t = torch.randn(n, V, generator=g)
+        return (t / t.std(unbiased=False)) * 0.9682458365518543
+
+    def _expand(self):
+        if self.decode_mode == 'lut':
+            return self.tlut
+        if self.decode_mode == 'quantlut':
+            return quantlut(self.tlut, self.L, self.tlut_bits)
+        return quantlut_sym(self.tlut, self.L, self.tlut_bits)
+
     def recons_lut(self):
-        self.lut = quantlut_sym(self.tlut, self.L, self.tlut_bits).T.contiguous()
+        if self.decode_mode not in _COMPUTED:
+            self.lut = self._expand().T.contiguous()
 
     def recons(self, encoded, **kwargs):
         return self.lut[:, encoded.int().to(self.lut.device)].to(encoded.device)
 
     def unpack_trellis(self, packed, T):
-        """Natural (non-kernel) packing -> (ntiles, T/V) states
-        (lib/codebook/bitshift.py:329-353), vectorised: state i is the 16-bit
-        window at bit offset i*K*V of the tile's circular bitstream."""
+        """Natural (non-kernel) packing -> (ntiles, T/V) int32 states
+        (lib/codebook/bitshift.py:329-353): state i is the 16-bit window at bit offset i*K*V of
+        the tile's circular bitstream.  Device tensors go through the HIP kernel; host tensors
+        (checkpoint conversion before upload) use the same window formula in torch."""
+        if packed.is_cuda:
+            return ops.unpack_trellis(packed.contiguous(), T, self.K, self.V)
         words = packed.view(torch.uint16).to(torch.int32).reshape(-1, T * self.K // 16)
         nxt = torch.roll(words, -1, dims=1)
         win = (words << 16) | nxt
@@ -76,10 +158,15 @@ class bitshift_codebook(nn.Module):
         w_idx, off = pos // 16, pos % 16
         return ((win[:, w_idx] >> (16 - off)) & 0xFFFF).to(torch.int32)
 
+    def pack_trellis(self, trellis):
+        """(ntiles, T/V) states -> natural packing, uint16 (lib/codebook/bitshift.py:294-327),
+        on the device that holds `trellis` (a GPU tensor is required)."""
+        return ops.pack_trellis(trellis.to(torch.int32).contiguous(), self.K, self.V)
+
     def quantize(self, *a, **k):
         raise NotImplementedError("quantisation (Viterbi) is outside the inference path")
 
-    viterbi = update = quantize_seq = pack_trellis = quantize
+    viterbi = update = quantize_seq = quantize
 
 
 class BitshiftLinear(nn.Module):
@@ -103,6 +190,15 @@ class BitshiftLinear(nn.Module):
         return self.cb.recons(unpacked_trellis).transpose(0, 1).transpose(1, 2).reshape(
             m // self.td_x, n // self.td_y, self.td_x, self.td_y).transpose(1, 2).reshape(m, n)
 
+    def get_hatW_natural(self, packed_trellis, m, n):
+        """Natural packing -> (m, n) in one launch for any decode mode: what
+        get_hatW(cb.unpack_trellis(.)) computes (lib/codebook/bitshift.py:329-381)."""
+        lut = self.cb.lut
+        if lut.dtype not in (torch.float16, torch.float32):
+            lut = lut.float()
+        lut = lut.to(packed_trellis.device).contiguous()
+        return ops.decode_natural(packed_trellis.contiguous(), lut, m, n, self.td_x, self.td_y, self.cb.K, self.V)
+
     def get_hatW_kernel(self, trellis, m, n):
         """Kernel-packed trellis -> (m, n) fp16 on the HIP decode kernel
         (lib/codebook/bitshift.py:383-387)."""
@@ -119,7 +215,7 @@ class BitshiftLinear(nn.Module):
         if self.has_kernel:
             hatW = self.get_hatW_kernel(packed_trellis, m, n)
         else:
-            hatW = self.get_hatW(self.cb.unpack_trellis(packed_trellis, self.td_x * self.td_y), m, n)
+            hatW = self.get_hatW_natural(packed_trellis, m, n)
         hatW = hatW.float() / self.scale
         if rcp == 1:
             self.hatW = matmul_hadU_cuda(
@@ -182,8 +278,10 @@ class BitshiftLinear(nn.Module):
             else:
                 y = ops.decompress_gemm(trellis.reshape(-1), xt, tl, m, n, self.cb.K, round_f16=True)
         else:
-            st = trellis if mode != 'eval' else self.cb.unpack_trellis(trellis, self.td_x * self.td_y)
-            hatW = self.get_hatW(st, m, n)
+            if mode == 'eval':
+                hatW = self.get_hatW_natural(trellis, m, n)
+            else:  # the owning module already turned the trellis into states
+                hatW = self.get_hatW(trellis, m, n)
             y = (xt.to(hatW.dtype) @ hatW.T).float()
 
         # ---- output transform: (H_R y / sqrt(m)) * SV * 32, cast

@@ -618,7 +618,7 @@ int choose_split(int m, int k, int bits, int cus) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 3; }
+int qtip_abi_version(void) { return 4; }
 
 const char* qtip_error_string(int code) {
   switch (code) {

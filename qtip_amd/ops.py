@@ -234,3 +234,77 @@ def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head
                                           _ptr(inv_freq), heads, kv_heads, head_dim, max_len,
                                           stream_ptr(qkv.device)), "qtip_decode_attention")
     return out
+
+
+# ---- packing tools ---------------------------------------------------------------------------
+
+def repack(packed, m, k, bits, to_kernel=True):
+    """Natural packing <-> kernel packing of a 16x16-tile, V=2 trellis (same shape and dtype out).
+    to_kernel=True is the re-pack of lib/algo/finetune.py:196-201, False its inverse
+    (lib/utils/kernel_decompress.py:19-24)."""
+    _check_packed(packed, m, k, bits)
+    out = torch.empty_like(packed)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_repack(_ptr(out), _ptr(packed), m, k, bits, 1 if to_kernel else 0,
+                                stream_ptr(packed.device)), "qtip_repack")
+    return out
+
+
+def _check_natural(packed, T, K, V):
+    require_cuda(packed, "packed", (torch.int16, torch.uint16))
+    if V not in (1, 2) or K * V > 16 or T % V or (T * K) % 16:
+        raise ValueError(f"unsupported natural packing T={T} K={K} V={V}")
+    nw = T * K // 16
+    if packed.numel() % nw:
+        raise ValueError(f"packed holds {packed.numel()} words, not a multiple of {nw} per tile")
+    return packed.numel() // nw
+
+
+def unpack_trellis(packed, T, K, V):
+    """Natural packing (ntiles, T*K/16) int16/uint16 -> (ntiles, T/V) int32 states
+    (lib/codebook/bitshift.py:329-353)."""
+    ntiles = _check_natural(packed, T, K, V)
+    states = torch.empty((ntiles, T // V), dtype=torch.int32, device=packed.device)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_unpack_trellis(_ptr(states), _ptr(packed), ntiles, T, K, V, stream_ptr(packed.device)),
+              "qtip_unpack_trellis")
+    return states
+
+
+def pack_trellis(states, K, V):
+    """(ntiles, T/V) states -> natural packing (ntiles, T*K/16) uint16
+    (lib/codebook/bitshift.py:294-327).  Raises, like the reference's assert, when consecutive
+    states do not overlap by 16 - K*V bits (this check synchronises with the device)."""
+    require_cuda(states, "states", torch.int32)
+    if states.dim() != 2:
+        raise ValueError("states must be (ntiles, T/V)")
+    ntiles, ns = states.shape
+    T = ns * V
+    if V not in (1, 2) or K * V > 16 or (T * K) % 16:
+        raise ValueError(f"unsupported natural packing T={T} K={K} V={V}")
+    packed = torch.empty((ntiles, T * K // 16), dtype=torch.uint16, device=states.device)
+    bad = torch.zeros(1, dtype=torch.int32, device=states.device)
+    with torch.cuda.device(states.device):
+        check(lib().qtip_pack_trellis(_ptr(packed), _ptr(states), ntiles, T, K, V, _ptr(bad),
+                                      stream_ptr(states.device)), "qtip_pack_trellis")
+    nbad = int(bad.item())
+    if nbad:
+        raise ValueError(f"pack_trellis: {nbad} consecutive state pairs are not a bitshift trellis walk")
+    return packed
+
+
+def decode_natural(packed, lut, m, n, td_x, td_y, K, V):
+    """Natural packing -> dense (m, n) in the dtype of `lut`, the expanded (V, 65536) table of the
+    codebook (fp16 or fp32): get_hatW(unpack_trellis(.)) of lib/codebook/bitshift.py:329-381."""
+    T = td_x * td_y
+    ntiles = _check_natural(packed, T, K, V)
+    if m % td_x or n % td_y or ntiles != (m // td_x) * (n // td_y) or td_y % V:
+        raise ValueError(f"packed does not describe a {m}x{n} matrix of {td_x}x{td_y} tiles")
+    require_cuda(lut, "lut", (torch.float16, torch.float32))
+    if lut.shape != (V, 65536) or lut.device != packed.device:
+        raise ValueError(f"lut must be ({V}, 65536) on {packed.device}")
+    out = torch.empty((m, n), dtype=lut.dtype, device=packed.device)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_decode_natural(_ptr(out), _ptr(packed), _ptr(lut), _DT[lut.dtype], m, n, td_x, td_y, K, V,
+                                        stream_ptr(packed.device)), "qtip_decode_natural")
+    return out

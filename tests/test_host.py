@@ -144,6 +144,8 @@ def test_quantiser_entry_points_raise():
     with pytest.raises(NotImplementedError):
         cb.quantize(None)
     with pytest.raises(NotImplementedError):
-        bitshift_codebook(16, 2, 1, 16, '1mad')
+        bitshift_codebook(12, 2, 1, 16, '1mad')  # only 16-bit state windows are built
+    with pytest.raises(ValueError):  # packing states needs device tensors
+        cb.pack_trellis(torch.zeros(1, 128, dtype=torch.int32))
     with pytest.raises(ValueError):
         BitshiftLinear(16, 16, 16, 5, 2, 9, 'quantlut_sym', has_kernel=True)
