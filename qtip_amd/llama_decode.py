@@ -35,14 +35,17 @@ class LlamaConfig:
         self.head_dim = hidden // heads
 
 
-def _qlinear(cfg, fin, fout, gen, device):
-    lin = QuantizedLinear(fin, fout, 16, 16, 16, cfg.K, 2, 9, 'quantlut_sym', dtype=torch.float16)
-    with torch.no_grad():
-        lin.trellis.copy_(torch.randint(-32768, 32768, lin.trellis.shape, dtype=torch.int16, generator=gen))
-        lin.tlut.copy_(torch.randn(512, 2, generator=gen).half())
-        lin.SU.copy_(torch.sign(torch.randn(fin, generator=gen) + 1e-5).half())
-        # decoded weights are ~N(0,1): scale so that the layer behaves like a 1/sqrt(fan_in) init
-        lin.SV.copy_(torch.sign(torch.randn(fout, generator=gen) + 1e-5) / math.sqrt(fin))
+def _qlinear(cfg, fin, fout, gen, device, K=None):
+    """A QuantizedLinear of the HYB code; seeded random contents when `gen` is given (the loader
+    passes None and fills the buffers from a checkpoint)."""
+    lin = QuantizedLinear(fin, fout, 16, 16, 16, K or cfg.K, 2, 9, 'quantlut_sym', dtype=torch.float16)
+    if gen is not None:
+        with torch.no_grad():
+            lin.trellis.copy_(torch.randint(-32768, 32768, lin.trellis.shape, dtype=torch.int16, generator=gen))
+            lin.tlut.copy_(torch.randn(512, 2, generator=gen).half())
+            lin.SU.copy_(torch.sign(torch.randn(fin, generator=gen) + 1e-5).half())
+            # decoded weights are ~N(0,1): scale so that the layer behaves like a 1/sqrt(fan_in) init
+            lin.SV.copy_(torch.sign(torch.randn(fout, generator=gen) + 1e-5) / math.sqrt(fin))
     return lin.to(device)
 
 
@@ -60,23 +63,51 @@ class RMSNorm(nn.Module):
 
 
 class DecoderLayer(nn.Module):
+    """fused=True: one quantized matrix for q/k/v and one for up/gate (the layout the reference's
+    README quotes its speed on).  fused=False: the seven separate projections of the reference's
+    model/llama.py (q_proj, k_proj, v_proj, o_proj, gate_proj, up_proj, down_proj), the layout of
+    its published checkpoints; a projection named in `skip` stays a dense fp16 nn.Linear."""
 
-    def __init__(self, cfg, gen, device):
+    def __init__(self, cfg, gen, device, fused=True, skip=(), K_v=None):
         super().__init__()
         d, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
         self.cfg = cfg
+        self.fused = fused
         self.input_norm = RMSNorm(d, cfg.eps).to(device)
         self.post_norm = RMSNorm(d, cfg.eps).to(device)
-        self.qkv = _qlinear(cfg, d, d + 2 * kvd, gen, device)
-        self.o = _qlinear(cfg, d, d, gen, device)
-        self.up_gate = _qlinear(cfg, d, 2 * cfg.ffn, gen, device)
-        self.down = _qlinear(cfg, cfg.ffn, d, gen, device)
+
+        def proj(name, fin, fout, K=None):
+            if name in skip:
+                return nn.Linear(fin, fout, bias=False, dtype=torch.float16, device=device)
+            return _qlinear(cfg, fin, fout, gen, device, K)
+
+        if fused:
+            self.qkv = proj('qkv', d, d + 2 * kvd)
+            self.up_gate = proj('up_gate', d, 2 * cfg.ffn)
+        else:
+            self.q_proj = proj('q', d, d)
+            self.k_proj = proj('k', d, kvd)
+            self.v_proj = proj('v', d, kvd, K_v)
+            self.gate_proj = proj('gate', d, cfg.ffn)
+            self.up_proj = proj('up', d, cfg.ffn)
+        self.o = proj('o', d, d)
+        self.down = proj('down', cfg.ffn, d)
+
+    def _qkv(self, h):
+        if self.fused:
+            return self.qkv(h)
+        return torch.cat([self.q_proj(h), self.k_proj(h), self.v_proj(h)], dim=-1)
+
+    def _gate_up(self, h):
+        if self.fused:
+            return self.up_gate(h)
+        return torch.cat([self.gate_proj(h), self.up_proj(h)], dim=-1)
 
     def forward(self, x, cos, sin, k_cache, v_cache, cache_position, attn_mask):
         cfg = self.cfg
         q_len = x.shape[1]
         h = self.input_norm(x)
-        qkv = self.qkv(h)
+        qkv = self._qkv(h)
         d, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
         q, k, v = qkv.split([d, kvd, kvd], dim=-1)
         q = q.view(1, q_len, cfg.heads, cfg.head_dim).transpose(1, 2)
@@ -95,33 +126,50 @@ class DecoderLayer(nn.Module):
         attn = attn.transpose(1, 2).reshape(1, q_len, d)
         x = x + self.o(attn)
         h = self.post_norm(x)
-        ug = self.up_gate(h)
+        ug = self._gate_up(h)
         gate, up = ug.split([cfg.ffn, cfg.ffn], dim=-1)
         x = x + self.down(F.silu(gate) * up)
         return x
 
     def decode_fused(self, x, k_cache, v_cache, pos, inv_freq):
-        """One new token, x (1, hidden) fp16: 13 launches (4 x [transform, matvec, transform] + attention)."""
+        """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
+        layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections."""
         cfg = self.cfg
         if not hasattr(self, "_fused"):
-            self._fused = [_FusedLinear(l) for l in (self.qkv, self.o, self.up_gate, self.down)]
-        qkv_l, o_l, ug_l, down_l = self._fused
-        qkv = qkv_l(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+            names = ('qkv', 'o', 'up_gate', 'down') if self.fused else \
+                ('q_proj', 'k_proj', 'v_proj', 'o', 'gate_proj', 'up_proj', 'down')
+            self._fused = {n: _FusedLinear(getattr(self, n)) for n in names}
+        f = self._fused
+        if self.fused:
+            qkv = f['qkv'](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+        else:
+            qkv = torch.cat([f[n](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+                             for n in ('q_proj', 'k_proj', 'v_proj')], dim=-1)
         attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
                                     cfg.head_dim)
-        x = o_l(attn.reshape(1, -1), residual=x)
-        ug = ug_l(x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
-        return down_l(ug, ops.PRE_SILU_MUL, residual=x)
+        x = f['o'](attn.reshape(1, -1), residual=x)
+        if self.fused:
+            ug = f['up_gate'](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+        else:
+            ug = torch.cat([f[n](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+                            for n in ('gate_proj', 'up_proj')], dim=-1)
+        return f['down'](ug, ops.PRE_SILU_MUL, residual=x)
 
 
 class _FusedLinear:
     """The three launches of a bs=1 QuantizedLinear with the neighbouring element-wise work of
     the decoder layer folded into the two transforms (RMSNorm or SiLU*up on the way in, the
-    residual addition on the way out)."""
+    residual addition on the way out).  A dense nn.Linear (a projection the checkpoint left
+    unquantized) gets the same interface on library kernels."""
 
     def __init__(self, lin):
-        dev = lin.trellis.device
         self.lin = lin
+        self.dense = isinstance(lin, nn.Linear)
+        if self.dense:
+            return
+        if not lin.has_kernel or int(lin.rcp) != 0:
+            raise NotImplementedError("fused decode needs kernel-packed HYB layers with rcp == 0")
+        dev = lin.trellis.device
         self.n, self.m, self.K = lin.in_features, lin.out_features, lin.K
         self.trellis = lin.trellis.reshape(-1)
         self.tlut = lin.tlut.data.reshape(-1).contiguous()
@@ -130,7 +178,19 @@ class _FusedLinear:
         self.bl = had_bits(lin.had_left, self.Kl, True, dev) if self.Kl > 1 else None
         self.br = had_bits(lin.had_right, self.Kr, False, dev) if self.Kr > 1 else None
 
+    def _dense(self, x, pre_mode, norm_weight, eps, residual):
+        if pre_mode == ops.PRE_RMSNORM:
+            h = x.float()
+            x = norm_weight * (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype)
+        elif pre_mode == ops.PRE_SILU_MUL:
+            gate, up = x.split(x.shape[-1] // 2, dim=-1)
+            x = F.silu(gate) * up
+        y = self.lin(x)
+        return y if residual is None else residual + y
+
     def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
+        if self.dense:
+            return self._dense(x, pre_mode, norm_weight, eps, residual)
         xt = ops.rht(x, order=self.Kl, had_bits=self.bl, pre=self.SU, scale=(self.n**-0.5) / 32.0,
                      out_dtype=torch.float16, pre_mode=pre_mode, norm_weight=norm_weight, eps=eps)
         parts = ops.decompress_matvec_parts(self.trellis, xt.reshape(-1), self.tlut, self.m, self.n, self.K)
@@ -145,15 +205,26 @@ def _rotate_half(x):
 
 
 class LlamaDecoder(nn.Module):
+    """gen=None (used by the checkpoint loader) leaves every tensor zero / identity."""
 
-    def __init__(self, cfg, max_cache_len, seed=0, device="cuda"):
+    def __init__(self, cfg, max_cache_len, seed=0, device="cuda", fused=True, skip=(), K_v=None, random_init=True):
         super().__init__()
         self.cfg = cfg
-        gen = torch.Generator().manual_seed(seed)
-        self.embed = (torch.randn(cfg.vocab, cfg.hidden, generator=gen) * 0.02).half().to(device)
-        self.layers = nn.ModuleList([DecoderLayer(cfg, gen, device) for _ in range(cfg.layers)])
+        self.fused = fused
+        gen = torch.Generator().manual_seed(seed) if random_init else None
+
+        def dense(rows, cols):
+            if gen is None:
+                return torch.zeros(rows, cols, dtype=torch.float16, device=device)
+            return (torch.randn(rows, cols, generator=gen) * 0.02).half().to(device)
+
+        self.embed = dense(cfg.vocab, cfg.hidden)
+        self.layers = nn.ModuleList([
+            DecoderLayer(cfg, gen, device, fused=fused,
+                         skip={n.split('_', 1)[1] for n in skip if n.split('_', 1)[0] == str(i)}, K_v=K_v)
+            for i in range(cfg.layers)])
         self.norm = RMSNorm(cfg.hidden, cfg.eps).to(device)
-        self.lm_head = (torch.randn(cfg.vocab, cfg.hidden, generator=gen) * 0.02).half().to(device)
+        self.lm_head = dense(cfg.vocab, cfg.hidden)
         self.max_cache_len = max_cache_len
         shape = (1, cfg.kv_heads, max_cache_len, cfg.head_dim)
         self.k_cache = [torch.zeros(shape, dtype=torch.float16, device=device) for _ in range(cfg.layers)]

@@ -1,0 +1,133 @@
+"""Checkpoint reader/writer for the reference's Hugging Face layout and the quantiser's per-layer
+dictionaries.  CPU tests cover the file format and the Wscale folding; the GPU tests run the
+loaded model."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from qtip_amd import checkpoint as C
+from qtip_amd.linear.quantized_linear import QuantizedLinear
+from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder
+
+
+def _tiny(device, skip=('1_k', '0_down'), seed=0, K_v=None):
+    cfg = LlamaConfig(hidden=256, heads=4, kv_heads=2, layers=2, ffn=512, vocab=96, K=2)
+    return LlamaDecoder(cfg, 64, seed=seed, device=device, fused=False, skip=skip, K_v=K_v)
+
+
+def _state(model):
+    return {k: (v.detach().cpu() if isinstance(v, torch.Tensor) else torch.tensor(v))
+            for k, v in C._targets(model).items()}
+
+
+@pytest.mark.parametrize("shard_bytes", [4 << 30, 100000])
+def test_save_load_round_trip_cpu(tmp_path, shard_bytes):
+    model = _tiny('cpu', K_v=3)
+    for layer in model.layers:  # skipped projections and norms get non-trivial values
+        layer.input_norm.weight.data.uniform_(0.5, 1.5)
+        for mod in layer.children():
+            if isinstance(mod, torch.nn.Linear):
+                mod.weight.data.normal_(0, 0.05)
+    C.save_llama(model, str(tmp_path), max_shard_bytes=shard_bytes)
+    files = sorted(os.listdir(tmp_path))
+    assert 'config.json' in files
+    if shard_bytes < 1 << 20:
+        assert 'model.safetensors.index.json' in files and sum(f.endswith('.safetensors') for f in files) > 1
+    cfg = json.load(open(tmp_path / 'config.json'))
+    assert cfg['quip_params']['skip_list'] == ['0_down', '1_k'] and cfg['quip_params']['K_v_proj'] == 3
+    loaded = C.load_llama(str(tmp_path), max_cache_len=64, device='cpu')
+    a, b = _state(model), _state(loaded)
+    assert a.keys() == b.keys()
+    for k in a:
+        assert a[k].dtype == b[k].dtype and torch.equal(a[k], b[k]), k
+    # reference key layout and dtypes
+    assert a['model.layers.0.self_attn.q_proj.trellis'].dtype == torch.int16
+    assert a['model.layers.0.self_attn.q_proj.SV'].dtype == torch.float32
+    assert a['model.layers.0.self_attn.v_proj.trellis'].shape == (8 * 16, 16 * 3)
+    assert 'model.layers.1.self_attn.k_proj.weight' in a and 'model.layers.0.mlp.down_proj.weight' in a
+
+
+def test_load_rejects_foreign_and_incomplete_checkpoints(tmp_path):
+    model = _tiny('cpu', skip=())
+    C.save_llama(model, str(tmp_path))
+    cfg = json.load(open(tmp_path / 'config.json'))
+    bad = dict(cfg)
+    bad['quip_params'] = dict(cfg['quip_params'], decode_mode='1mad')
+    json.dump(bad, open(tmp_path / 'config.json', 'w'))
+    with pytest.raises(NotImplementedError):
+        C.load_llama(str(tmp_path), 64, 'cpu')
+    bad = {k: v for k, v in cfg.items() if k != 'quip_params'}
+    json.dump(bad, open(tmp_path / 'config.json', 'w'))
+    with pytest.raises(ValueError):
+        C.load_llama(str(tmp_path), 64, 'cpu')
+    bad = dict(cfg, num_hidden_layers=3)  # tensors of a third layer are missing
+    json.dump(bad, open(tmp_path / 'config.json', 'w'))
+    with pytest.raises(KeyError):
+        C.load_llama(str(tmp_path), 64, 'cpu')
+    bad = dict(cfg, intermediate_size=1024)
+    json.dump(bad, open(tmp_path / 'config.json', 'w'))
+    with pytest.raises(ValueError):
+        C.load_llama(str(tmp_path), 64, 'cpu')
+
+
+@pytest.mark.parametrize("rcp", [None, 0, 1, 2])
+def test_unpack_quip_folds_wscale(rcp):
+    """lib/utils/data_utils.py:281-307: Wscale goes into SV (plain / column-parallel, per shard for
+    rcp 2) or into SU per shard (row-parallel, rcp 1)."""
+    fin, fout, shards = 256, 128, 8
+    g = torch.Generator().manual_seed(1)
+    lin = QuantizedLinear(fin, fout, 16, 16, 16, 2, 2, 9, 'quantlut_sym')
+    SU = torch.sign(torch.randn(fin, generator=g)).half()
+    SV = torch.sign(torch.randn(fout, generator=g)).half()
+    saved = dict(trellis=torch.randint(-32768, 32768, lin.trellis.shape, dtype=torch.int16, generator=g),
+                 tlut=torch.randn(512, 2, generator=g), SU=SU, SV=SV)
+    if rcp in (1, 2):
+        saved['Wscale'] = torch.rand(shards, generator=g) + 0.5
+    else:
+        saved['Wscale'] = torch.tensor(0.37)
+    if rcp is not None:
+        saved['rcp'] = torch.tensor(rcp)
+        saved['tp_rank'] = torch.tensor(shards)
+    C.unpack_quip(lin, saved)
+    assert torch.equal(lin.trellis, saved['trellis'])
+    assert torch.equal(lin.tlut.data, saved['tlut'].half())
+    w = saved['Wscale'].float()
+    if rcp == 1:
+        assert torch.equal(lin.SU.float(), (SU.float() * w.repeat_interleave(fin // shards)).half().float())
+        assert torch.equal(lin.SV, SV.float())
+    elif rcp == 2:
+        assert torch.equal(lin.SU, SU)
+        assert torch.equal(lin.SV, SV.float() * w.repeat_interleave(fout // shards))
+    else:
+        assert torch.equal(lin.SU, SU)
+        assert torch.equal(lin.SV, SV.float() * w)
+    if rcp is not None:
+        assert int(lin.rcp) == rcp and int(lin.tp_rank) == shards
+
+
+@pytest.mark.gpu
+def test_loaded_model_runs_like_the_original(tmp_path):
+    from qtip_amd.llama_decode import generate
+    dev = torch.device('cuda:0')
+    model = _tiny(dev, skip=('1_k',), seed=3)
+    C.save_llama(model, str(tmp_path))
+    loaded = C.load_llama(str(tmp_path), max_cache_len=64, device=dev)
+    ids = torch.randint(0, 96, (1, 9), generator=torch.Generator().manual_seed(0)).to(dev)
+    pos = torch.arange(9, device=dev)
+    with torch.no_grad():
+        a = model(ids, pos)
+        b = loaded(ids, pos)
+    assert torch.equal(a, b)
+    # fused transforms on the separate-projection layout follow the module path
+    with torch.no_grad():
+        tok = torch.tensor([[5]], device=dev)
+        p = torch.tensor([9], device=dev)
+        ref = model(tok, p)
+        got = loaded.decode_fused(tok, p)
+    err = (got - ref).abs().max() / ref.abs().max()
+    assert err < 2e-2
+    out, _, _ = generate(loaded, ids, 6, use_graph=True, fused=True)
+    assert out.shape == (1, 6)
