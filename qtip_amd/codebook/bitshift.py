@@ -247,6 +247,9 @@ class BitshiftLinear(nn.Module):
             self.cb.recons_lut()
         rcp = int(rcp)
         tp_rank = int(tp_rank)
+        if torch.is_grad_enabled() and (input.requires_grad or SU.requires_grad or SV.requires_grad):
+            return self._forward_autograd(input, trellis, SU, SV, had_left, had_right, K_left, K_right, rcp,
+                                          tp_rank, mode)
         dev = input.device
         x = input.reshape(-1, n)
         bs = x.shape[0]
@@ -302,6 +305,31 @@ class BitshiftLinear(nn.Module):
                          scale=mm**-0.5, out_dtype=torch.float32).reshape(bs, m)
             out = (yt.to(SV.device) * (SV * self.scale)).to(input.dtype)
         return out.view(*input.shape[:-1], m)
+
+
+    def _forward_autograd(self, input, trellis, SU, SV, had_left, had_right, K_left, K_right, rcp, tp_rank, mode):
+        """The same forward as a chain of differentiable steps, as the reference runs it when
+        fine-tuning (lib/codebook/bitshift.py:428-472): gradients reach the input and the sign
+        vectors SU / SV; the trellis is fixed and the table gets no gradient on the kernel path
+        (BitshiftLinearKernelAG returns None for it, :491-505)."""
+        n, m = len(SU), len(SV)
+        x = input.reshape(-1, n).to(torch.float32) * SU
+        if rcp == 1:
+            x = matmul_hadUt_cuda(x.reshape(-1, n // tp_rank), had_left, K_left).reshape(x.shape) / self.scale
+        else:
+            x = matmul_hadUt_cuda(x, had_left, K_left) / self.scale
+        if self.has_kernel:
+            x = BitshiftLinearKernelAG.apply(x, trellis, m, n, self.cb.L, self.cb.tlut_bits, self.cb.K, self.V,
+                                             self.cb.lut).float()
+        else:
+            hatW = self.get_hatW_natural(trellis, m, n) if mode == 'eval' else self.get_hatW(trellis, m, n)
+            x = (x.to(hatW.dtype) @ hatW.T).float()
+        if rcp == 2:
+            x = matmul_hadU_cuda(x.reshape(-1, m // tp_rank), had_right, K_right).reshape(x.shape)
+        else:
+            x = matmul_hadU_cuda(x, had_right, K_right)
+        x = x.to(SV.device) * (SV * self.scale)
+        return x.view(*input.shape[:-1], m).to(input.dtype)
 
 
 class BitshiftLinearKernelAG(torch.autograd.Function):

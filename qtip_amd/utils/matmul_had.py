@@ -101,14 +101,37 @@ def hadamard(x: torch.Tensor, scale: float) -> torch.Tensor:
     return ops.rht(x.contiguous(), scale=scale)
 
 
-def matmul_hadU_cuda(X, hadK, K, transpose=False):
-    """(H_K (x) H_{n/K}) X / sqrt(n) along the last axis (lib/utils/matmul_had.py:105-115)."""
+class _HadamardFn(torch.autograd.Function):
+    """y = (H_K (x) H_{n/K}) x / sqrt(n) with the gradient the reference gets from the autograd
+    support of its Walsh-Hadamard package plus the dense hadK matmul: the transform is linear and
+    orthonormal, so grad_x = (H_K^T (x) H_{n/K}) grad_y / sqrt(n) - the same kernel with the
+    order-K table transposed."""
+
+    @staticmethod
+    def forward(ctx, X, hadK, K, transpose):
+        ctx.hadK, ctx.K, ctx.transpose = hadK, K, transpose
+        return _hadU(X, hadK, K, transpose)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return _hadU(grad.contiguous(), ctx.hadK, ctx.K, not ctx.transpose), None, None, None
+
+
+def _hadU(X, hadK, K, transpose):
     n = X.shape[-1]
     if K == 1:
         return torch.ops.hadamard.hadamard(X.contiguous(), n**(-0.5))
     x = X if X.dtype in (torch.float16, torch.float32) else X.float()
     out = ops.rht(x.contiguous(), order=K, had_bits=had_bits(hadK, K, transpose, X.device), out_dtype=x.dtype)
     return out.to(X.dtype).reshape(X.shape)
+
+
+def matmul_hadU_cuda(X, hadK, K, transpose=False):
+    """(H_K (x) H_{n/K}) X / sqrt(n) along the last axis (lib/utils/matmul_had.py:105-115);
+    differentiable with respect to X."""
+    if torch.is_grad_enabled() and X.requires_grad:
+        return _HadamardFn.apply(X, hadK, K, transpose)
+    return _hadU(X, hadK, K, transpose)
 
 
 def matmul_hadUt_cuda(X, hadK, K):
