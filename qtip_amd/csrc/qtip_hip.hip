@@ -416,12 +416,33 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
   __syncthreads();
 
   // activations: lane (batch row a of tile nb, K group g) reads x[b][128*wl + 32*g + 16*kh + 0..15]
-  const uint16_t* xrow[NB];
+  // through a buffer descriptor that ends with the last batch row: the lanes of a ragged last
+  // wave-load (columns past k) and padding items get an offset past the end and read zeros,
+  // which cancel whatever those lanes decode.  The loads for item i+1 are issued before item i
+  // is decoded, so they have a whole stage to arrive.
+  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(x), 0, (int)((size_t)batch * k * 2), 0x00020000);
+  uint32_t xvoff[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int bb = 16 * nb + a;
-    xrow[nb] = x + (size_t)(bb < batch ? bb : 0) * k + 32 * g;
+    xvoff[nb] = (uint32_t)(bb < batch ? bb : 0) * (uint32_t)k * 2u + 64u * g;
   }
+  u32x4 xbuf[DEPTH][2][NB][2];  // [stage][kh][nb][low / high 16 bytes]
+  auto issue_x = [&](int d, int cj, bool item_ok) {
+    const int wl = wave + cj * kGemmWaves;
+    const bool ok = item_ok && cj < nvj && 128 * wl + 32 * g < k;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const uint32_t vo = ok ? xvoff[nb] : 0x7FFFFFC0u;
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) {
+        xbuf[d][kh][nb][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, vo + 32u * kh, (uint32_t)wl * 256u, 0);
+        xbuf[d][kh][nb][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, vo + 32u * kh + 16u, (uint32_t)wl * 256u, 0);
+      }
+    }
+  };
+  issue_x(0, 0, T > 0);
 
   float4_t acc[2][2][2][NB];  // [mh][rh][column half][batch tile]
 #pragma unroll
@@ -431,30 +452,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
+      issue_x((d + 1) % DEPTH, c_j + 1 == npw ? 0 : c_j + 1, t + d + 1 < T);
       if (t + d < T && c_j < nvj) {
-        const int wl = wave + c_j * kGemmWaves;
-        // activations first (their latency hides behind the decode)
-        u32x4 xa[2][NB][2];  // [kh][nb][low / high 16 bytes]
-        const bool in_k = 128 * wl + 32 * g < k;  // false only in the lanes of a ragged last wave-load
-        const size_t xo = in_k ? (size_t)wl * 128 : 0;
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const u32x4* px = reinterpret_cast<const u32x4*>(xrow[nb] + xo + 16 * kh);
-            xa[kh][nb][0] = px[0];
-            xa[kh][nb][1] = px[1];
-          }
-        if (!in_k) {
-          // columns past k: zero activations cancel whatever the lane decodes
-#pragma unroll
-          for (int kh = 0; kh < 2; ++kh)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              xa[kh][nb][0] = u32x4{0u, 0u, 0u, 0u};
-              xa[kh][nb][1] = u32x4{0u, 0u, 0u, 0u};
-            }
-        }
+        auto& xa = xbuf[d];
         uint32_t P[16], W[32];
         packed_states<K>(buf[d], P);
 #pragma unroll
