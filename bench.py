@@ -15,6 +15,8 @@ Prints ONE JSON line:  value = packed bytes streamed per second (GB/s), plus
                 oracle/torch_cpu_path.py) on a bounded sample, same host
   shapes        per-matrix kernel time / GB/s / fraction of 8 TB/s
   layer         whole BitshiftLinear.forward (RHT-in + matvec + RHT-out) per matrix
+  gemm_4bit     batched decompress-GEMM (batch 8/16/32) time, stream GB/s, TFLOP/s
+  e2e_decode    greedy decode tok/s of a random-init 7B-architecture 2-bit model
 """
 import argparse
 import json
@@ -195,6 +197,34 @@ def main():
             del gr
         result["shapes"] = per
         result["layer"] = layer
+
+        # batched decompress-GEMM on the matrix cores: 4-bit weights, batch 8 / 16 / 32
+        gemm = {}
+        for m, k in ((28672, 8192), (8192, 28672)):
+            nbytes = m * k * 4 // 8
+            base = torch.randint(-32768, 32768, (m * k * 4 // 16,), dtype=torch.int16, generator=g).to(dev)
+            pk4 = [base] + [torch.roll(base, 4099 * c) for c in range(1, 6)]
+            for B in (8, 16, 32):
+                X = torch.randn(B, k, generator=g).half().to(dev)
+                gr = capture(lambda: [ops.decompress_gemm(pk4[i % 6], X, tlut, m, k, 4) for i in range(12)])
+                us = timed(gr, 3) * 1e6 / 12
+                tf = 2.0 * m * k * B / us / 1e6
+                gemm[f"{m}x{k}_b{B}"] = {"us": round(us, 2), "stream_GBps": round(nbytes / us / 1e3, 1),
+                                         "TFLOPs": round(tf, 1), "frac_mfma_f16_peak": round(tf / 2500.0, 4)}
+                del gr
+            del pk4, base
+        result["gemm_4bit"] = gemm
+
+        # end-to-end greedy decode, random-init Llama-2-7B architecture, every linear 2-bit
+        from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+        model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev)
+        prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
+        _, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
+        result["e2e_decode"] = {"model": "Llama-2-7B architecture, random init, 2-bit HYB, fused qkv and up/gate",
+                                "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1),
+                                "ms_per_token": round(1e3 / tps, 3)}
+        del model
+        torch.cuda.empty_cache()
 
     # ---- CPU baseline (bounded sample) -------------------------------------
     if not args.no_cpu:
