@@ -46,7 +46,10 @@ def main():
                     help="restrict the set to one of its matrices (qkv, o, up_gate, down): used for per-kernel "
                          "counter runs under rocprofv3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer timings")
+    ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
+    ap.add_argument("--extras", default="shapes,layer,gemm,e2e",
+                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, e2e "
+                         "(counter runs under rocprofv3 pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs)")
@@ -171,7 +174,8 @@ def main():
     }
 
     # ---- per-shape kernel times and whole-layer times ---------------------
-    if not args.no_extras:
+    extras = set() if args.no_extras else set(args.extras.split(","))
+    if extras & {"shapes", "layer"}:
         from qtip_amd.codebook.bitshift import BitshiftLinear
         from qtip_amd.utils import matmul_had as mh
         per, layer = {}, {}
@@ -198,6 +202,7 @@ def main():
         result["shapes"] = per
         result["layer"] = layer
 
+    if "gemm" in extras:
         # batched decompress-GEMM on the matrix cores: 4-bit weights, batch 8 / 16 / 32
         gemm = {}
         for m, k in ((28672, 8192), (8192, 28672)):
@@ -215,6 +220,7 @@ def main():
             del pk4, base
         result["gemm_4bit"] = gemm
 
+    if "e2e" in extras:
         # end-to-end greedy decode, random-init Llama-2-7B architecture, every linear 2-bit
         from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
         model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev)
