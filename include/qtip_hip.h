@@ -53,15 +53,16 @@ const char* qtip_error_string(int code);
 int qtip_decode(void* out_f16, const void* packed, const void* tlut,
                 int m, int k, int bits, void* stream);
 
-/* Number of k splits S (>= 1) the matvec uses for this shape on the current
- * device: small m cannot fill 256 CUs with 32-row blocks alone, so the k
- * dimension is cut into S ranges whose partial sums are added afterwards in a
- * fixed order.  Returns 0 for an unsupported shape. */
+/* Number of k splits S (>= 1) recommended for qtip_decompress_matvec_parts on this shape and
+ * device: small m cannot fill 256 CUs with 32-row blocks alone, so the k dimension is cut into
+ * S ranges whose partial sums the consumer adds in a fixed order.  Returns 0 for an
+ * unsupported shape. */
 int qtip_matvec_split(int m, int k, int bits);
 
-/* Bytes of scratch qtip_decompress_matvec wants for this shape: S*m floats
- * when S > 1, else 0.  The scratch needs no initialisation.  Calls that share
- * one scratch buffer must not overlap in time. */
+/* Bytes of scratch qtip_decompress_matvec wants for this shape: S'*m floats when it splits k,
+ * else 0 (S' is chosen with the cost of the extra summing launch included, so it is 1 for most
+ * shapes).  The scratch needs no initialisation.  Calls that share one scratch buffer must not
+ * overlap in time. */
 size_t qtip_matvec_workspace_bytes(int m, int k, int bits);
 
 /* bs=1 decompress + matvec: out[m] (fp32) = hatW[m][k] . x[k] (fp16), fp32

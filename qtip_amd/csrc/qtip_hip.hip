@@ -593,8 +593,13 @@ int check_common(const void* a, const void* b, const void* c, const void* d, int
   return QTIP_OK;
 }
 
-// k split so that (m/32)*S units fill the machine evenly
-int choose_split(int m, int k, int bits, int cus) {
+// k split S for the shape.  Cost model in units of one wave-load per wave slot (fitted to
+// measured launch times of the 7B / 70B shapes): a workgroup walks `rounds` units of nwl/S
+// wave-loads, each unit carries a fixed cost (flush, barrier, pipeline refill), a launch never
+// takes less than the latency of its first stages, and when the caller wants the summed vector
+// (not the parts) a split costs one more small launch.
+int choose_split(int m, int k, int bits, int cus, bool summed) {
+  (void)bits;
   const int nrb = m >> 5;
   const int nwl = ((k >> 5) + 3) >> 2;
   int best = 1;
@@ -603,9 +608,10 @@ int choose_split(int m, int k, int bits, int cus) {
     if (nwl / S < kWaves && S > 1) break;  // keep at least one wave-load per wave
     const long units = (long)nrb * S;
     const long rounds = (units + cus - 1) / cus;
-    // cost: rounds * (unit bytes + fixed per-unit overhead expressed in bytes)
-    const double unit_bytes = (double)nwl / S * 512.0 * bits;
-    const double cost = rounds * (unit_bytes + 12288.0 + (S > 1 ? 4096.0 : 0.0));
+    const double per_unit = (double)nwl / S + 12.0 + (S > 1 ? 4.0 : 0.0);
+    double cost = rounds * per_unit;
+    if (cost < 60.0) cost = 60.0;
+    if (S > 1 && summed) cost += 53.0;
     if (cost < best_cost * 0.97) {
       best_cost = cost;
       best = S;
@@ -661,11 +667,14 @@ int qtip_matvec_split(int m, int k, int bits) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
   DeviceInfo& di = device_info();
   if (!di.ok) return 0;
-  return choose_split(m, k, bits, di.cus);
+  return choose_split(m, k, bits, di.cus, false);
 }
 
 size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
-  const int S = qtip_matvec_split(m, k, bits);
+  if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return 0;
+  const int S = choose_split(m, k, bits, di.cus, true);
   return S > 1 ? (size_t)S * m * sizeof(float) : 0;
 }
 
@@ -726,7 +735,7 @@ int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, co
   if (rc) return rc;
   int S = 1;
   if (workspace) {
-    S = choose_split(m, k, bits, device_info().cus);
+    S = choose_split(m, k, bits, device_info().cus, true);
     if (S > 1 && workspace_bytes < (size_t)S * m * sizeof(float)) return QTIP_E_WORKSPACE;
     if (!aligned16(workspace)) return QTIP_E_ALIGN;
   }
