@@ -257,6 +257,248 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Vectorised form (pp a multiple of 8, 16-byte aligned rows): the same mix + transform, but a
+// thread loads 8 consecutive columns of a row j with one 16-byte load (two for fp32 input), so
+// a vector costs n/8192 load instructions per thread instead of n/1024 two-byte gathers - the
+// scalar form is bound by the address rate of the vector-memory unit, not by bytes.
+//   thread t: column group cg = t % (pp/8), row group jg = t / (pp/8); rows j = jg, jg + JG, ...
+//   z[e] (8 columns) accumulates over the thread's rows, lanes that share cg are summed with
+//   cross-lane adds, the 16 waves' partial vectors (8 row groups for pp = 1024) meet in LDS,
+//   thread c < pp then owns column c for the pp-point transform as in the scalar form.
+// The per-output operands (post, residual) are fetched at the start, so their latency (they are
+// cold in the decode loop: every layer has its own) overlaps the loads of the vector.
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <typename TIn>
+struct Raw8;
+template <>
+struct Raw8<_Float16> {
+  uint4 a;
+  __device__ __forceinline__ void load(const _Float16* p) { a = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void get(float v[8]) const {
+    const half8v h = __builtin_bit_cast(half8v, a);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (float)h[e];
+  }
+};
+template <>
+struct Raw8<float> {
+  float4v a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const float4v*>(p);
+    b = *reinterpret_cast<const float4v*>(p + 4);
+  }
+  __device__ __forceinline__ void get(float v[8]) const {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = a[e];
+      v[4 + e] = b[e];
+    }
+  }
+};
+
+template <typename TIn, typename TOut, int CH, bool FUSED>
+__global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P) {
+  __shared__ __align__(16) float red[8192];  // partial vectors [NP][pp], then the exchange buffer of the transform
+  __shared__ float wsum[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int A = 1 << P.logA;
+  const int iK = blockIdx.x >> P.logA, iA = blockIdx.x & (A - 1);
+  const size_t r = blockIdx.y;
+  const int n = P.n, pp = P.pp, order = P.order;
+  const TIn* src = reinterpret_cast<const TIn*>(P.in) + r * P.in_row_stride;
+  const int OT = order << P.logA;
+  const int CG = pp >> 3;            // column groups of 8 (power of two, 1 .. 128)
+  const int JG = kRhtThreads / CG;   // row groups
+  int lcg = 0;
+  while ((1 << lcg) < CG) ++lcg;
+  const int cg = tid & (CG - 1), jg = tid >> lcg;
+  const int pre_mode = FUSED ? P.pre_mode : PRE_NONE;
+
+  // ---- this thread's output element and its operands
+  const bool active = tid < pp;
+  const int W = pp > 64 ? pp >> 6 : 1;  // waves holding the row in the transform
+  int cfin = tid;
+  if (W > 1) {
+    const int wv = tid >> 6;
+    cfin = 64 * (lane & (W - 1)) + (lane / W) + (64 / W) * wv;  // after the transposed read
+  }
+  const size_t oidx = ((size_t)iK * A + iA) * pp + cfin;
+  float postv = 1.f, resv = 0.f;
+  if (active) {
+    if (P.post) postv = P.post[oidx];
+    if (FUSED && P.residual) resv = (float)P.residual[r * (size_t)n + oidx];
+  }
+
+  float z[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) z[e] = 0.f;
+  const int npass = ((OT + JG - 1) / JG + CH - 1) / CH;  // the same for every thread (barriers inside)
+  for (int pass = 0; pass < npass; ++pass) {
+    const int j0 = jg + pass * JG * CH;
+    Raw8<TIn> xr[CH], ar[FUSED ? CH : 1];
+    Raw8<_Float16> sr[CH], nw[FUSED ? CH : 1];
+    uint32_t br[CH];
+    bool ok[CH];
+    size_t base[CH];
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      ok[q] = j < OT;
+      base[q] = (size_t)(ok[q] ? j : 0) * pp + 8 * cg;
+      xr[q].load(src + base[q]);
+      br[q] = 0;
+    }
+    if (P.pre) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) sr[q].load(P.pre + base[q]);
+    }
+    if (order > 1) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        const int j = j0 + q * JG;
+        const unsigned bit = (unsigned)((ok[q] ? j : 0) >> P.logA) * order + iK;
+        br[q] = (P.had_bits[bit >> 5] >> (bit & 31)) & 1u;
+      }
+    }
+    if (FUSED && pre_mode == PRE_RMSNORM) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) nw[q].load(P.norm_w + base[q]);
+    }
+    if (FUSED && pre_mode == PRE_SILU_MUL) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) ar[q].load(src + (size_t)n + base[q]);
+    }
+    float v[CH][8];
+#pragma unroll
+    for (int q = 0; q < CH; ++q) xr[q].get(v[q]);
+    for (int w = 1; w < P.in_parts; ++w) {
+      Raw8<TIn> pr[CH];
+#pragma unroll
+      for (int q = 0; q < CH; ++q) pr[q].load(src + w * P.part_stride + base[q]);
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        float t[8];
+        pr[q].get(t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] += t[e];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < CH; ++q)
+      if (!ok[q]) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] = 0.f;
+      }
+    // ---- element-wise prologue
+    if (FUSED && pre_mode == PRE_RMSNORM) {
+      float ss = 0.f;
+#pragma unroll
+      for (int q = 0; q < CH; ++q)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[q][e] * v[q][e];
+      ss = wave_sum(ss);
+      if (lane == 0) wsum[wave] = ss;
+      __syncthreads();
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) tot += wsum[w];
+      const float rs = __builtin_amdgcn_rsqf(tot / (float)n + P.eps);
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        float wn[8];
+        nw[q].get(wn);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] = (float)(_Float16)(wn[e] * (float)(_Float16)(v[q][e] * rs));
+      }
+    } else if (FUSED && pre_mode == PRE_SILU_MUL) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        float up[8];
+        ar[q].get(up);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float g = v[q][e];
+          const float sl = (float)(_Float16)(g / (1.f + __expf(-g)));
+          v[q][e] = (float)(_Float16)(sl * up[e]);
+        }
+      }
+    }
+    // ---- mix
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      const uint32_t sg = (br[q] ^ ((uint32_t)__builtin_popcount(iA & (j & (A - 1))) & 1u)) << 31;
+      float f[8];
+      if (P.pre) {
+        sr[q].get(f);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = 1.f;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        z[e] += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[q][e] * f[e]) ^ sg);
+    }
+  }
+  // ---- lanes that share a column group (they differ in lane bits lcg .. 5)
+#pragma unroll
+  for (int b = 0; b < 6; ++b) {
+    if (b >= lcg) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z[e] += lane_xor(z[e], b);
+    }
+  }
+  // ---- partial vectors to LDS: one per wave (CG <= 64) or one per row group (CG = 128)
+  const int NP = CG <= 64 ? 16 : JG;
+  const int part = CG <= 64 ? wave : jg;
+  if (CG > 64 || lane < CG) {
+    float4v* dst = reinterpret_cast<float4v*>(red + part * pp + 8 * cg);
+    dst[0] = float4v{z[0], z[1], z[2], z[3]};
+    dst[1] = float4v{z[4], z[5], z[6], z[7]};
+  }
+  __syncthreads();
+  float y = 0.f;
+  if (active) {
+    for (int q = 0; q < NP; ++q) y += red[q * pp + tid];
+  }
+  __syncthreads();
+  // ---- pp-point transform of column tid
+  int nb0 = 0;
+  while (nb0 < 6 && (1 << nb0) < pp) ++nb0;
+  if (active) {
+    y = wht_lanes(y, nb0, lane);
+    if (W > 1) red[tid] = y;
+  }
+  if (W > 1) {
+    __syncthreads();
+    if (active) {
+      y = red[cfin];
+      int nb = 0;
+      while ((1 << nb) < W) ++nb;
+      y = wht_lanes(y, nb, lane);
+    }
+  }
+  if (active) {
+    const float o = y * P.scale * postv;
+    TOut* op = reinterpret_cast<TOut*>(P.out) + r * (size_t)n + oidx;
+    if (FUSED && P.residual) *op = (TOut)(_Float16)(resv + (float)(_Float16)o);
+    else *op = (TOut)o;
+  }
+}
+
+template <typename TI, typename TO, bool FUSED>
+int launch_rht_vec(const RhtParams& P, dim3 grid, long loads, hipStream_t st) {
+  // a prologue needs the whole row in one pass
+  if (FUSED && P.pre_mode == PRE_RMSNORM && loads > 4) return QTIP_E_SHAPE;
+  if (loads <= 1) rht_vec_kernel<TI, TO, 1, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
+  else if (loads <= 2) rht_vec_kernel<TI, TO, 2, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
+  else rht_vec_kernel<TI, TO, 4, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
+  return (int)hipGetLastError();
+}
+
 template <typename TI, typename TO, bool FUSED>
 int launch_rht_l(const RhtParams& P, dim3 grid, long loads, int ri, hipStream_t st) {
   // a prologue needs the whole row in one pass
@@ -296,18 +538,39 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
     ++logA;
   }
   const long OT = (long)order << logA;
-  const int JG = kRhtThreads / pp;
-  const long loads = (OT + JG - 1) / JG;
   P.logA = logA;
   P.pp = pp;
+  hipStream_t st = (hipStream_t)stream;
+  const bool fused = P.pre_mode != PRE_NONE || P.residual != nullptr;
+  if (fused && out_dtype != QTIP_F16) return QTIP_E_DTYPE;  // fused forms exist for the combinations the decode loop uses
+  // vectorised form: 8 columns per thread, 16-byte loads
+  const size_t esz = in_dtype == QTIP_F16 ? 2 : 4;
+  // (vectors of up to 4096 elements stay on the scalar form: it has fewer phases and its few
+  // loads per thread are not the limit there)
+  const bool vec_ok = pp >= 8 && n > 4096 && (reinterpret_cast<uintptr_t>(P.in) & 15u) == 0 &&
+                      ((P.in_row_stride * esz) & 15u) == 0 && ((P.part_stride * esz) & 15u) == 0 &&
+                      (!P.pre || (reinterpret_cast<uintptr_t>(P.pre) & 15u) == 0) &&
+                      (!P.norm_w || (reinterpret_cast<uintptr_t>(P.norm_w) & 15u) == 0) &&
+                      !(P.pre_mode == PRE_SILU_MUL && ((size_t)n * esz & 15u));
+  if (vec_ok) {
+    const int JGv = kRhtThreads / (pp >> 3);
+    const long vloads = (OT + JGv - 1) / JGv;
+    dim3 vgrid((unsigned)OT, rows);
+    if (fused) {
+      if (in_dtype == QTIP_F16) return launch_rht_vec<_Float16, _Float16, true>(P, vgrid, vloads, st);
+      return launch_rht_vec<float, _Float16, true>(P, vgrid, vloads, st);
+    }
+    if (in_dtype == QTIP_F16 && out_dtype == QTIP_F16) return launch_rht_vec<_Float16, _Float16, false>(P, vgrid, vloads, st);
+    if (in_dtype == QTIP_F16 && out_dtype == QTIP_F32) return launch_rht_vec<_Float16, float, false>(P, vgrid, vloads, st);
+    if (in_dtype == QTIP_F32 && out_dtype == QTIP_F16) return launch_rht_vec<float, _Float16, false>(P, vgrid, vloads, st);
+    return launch_rht_vec<float, float, false>(P, vgrid, vloads, st);
+  }
+  const int JG = kRhtThreads / pp;
+  const long loads = (OT + JG - 1) / JG;
   // large table orders: four rows of the mix per workgroup
   const int ri = (logA == 0 && order >= 64 && order % 4 == 0 && 4 * pp <= kRhtThreads && JG > 1) ? 4 : 1;
   dim3 grid((unsigned)(OT / ri), rows);
-  hipStream_t st = (hipStream_t)stream;
-  const bool fused = P.pre_mode != PRE_NONE || P.residual != nullptr;
   if (fused) {
-    // fused forms exist for the two combinations the decode loop uses
-    if (out_dtype != QTIP_F16) return QTIP_E_DTYPE;
     if (in_dtype == QTIP_F16) return launch_rht_l<_Float16, _Float16, true>(P, grid, loads, ri, st);
     return launch_rht_l<float, _Float16, true>(P, grid, loads, ri, st);
   }
