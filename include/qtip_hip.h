@@ -87,15 +87,21 @@ int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x
                                  const void* tlut, int m, int k, int bits, int nparts,
                                  void* stream);
 
+/* Bytes of scratch qtip_decompress_gemm wants for this shape (0 when it does not split k). */
+size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch);
+
 /* Batched decompress + GEMM on the matrix cores:
  * out[batch][m] = x[batch][k] (fp16) . hatW[m][k]^T, fp32 accumulate.
  * If round_f16 != 0 every result is rounded to fp16 and widened again, which
  * is what the reference's fp16 GEMM output followed by .float() yields.
  * Replaces BitshiftLinearKernelAG.forward = decode_compressed + input.half() @ hatW.T
- * (lib/codebook/bitshift.py:476-489).  1 <= batch <= 65535. */
+ * (lib/codebook/bitshift.py:476-489).  1 <= batch <= 65535.
+ * Matrices with few rows are also cut along k; the fp32 partial results then pass through
+ * `workspace` (qtip_gemm_workspace_bytes, no initialisation needed, 16-byte aligned) and one
+ * more small launch adds them in a fixed order.  workspace may be NULL: k is then never split. */
 int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16,
                          const void* tlut, int m, int k, int bits, int batch,
-                         int round_f16, void* stream);
+                         int round_f16, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Randomised Hadamard transform of `rows` vectors of length n = order * p
  * (p a power of two, order 1 or a table order):

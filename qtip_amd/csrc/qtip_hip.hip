@@ -367,160 +367,245 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ out,
 // core's work, which is free here (the kernel is bound by the decode), and
 // needs no data movement between decode and MFMA: the table lookups land in
 // the operand registers.
+//
+// Activations are shared through LDS: a workgroup (8 waves) works on 4 consecutive 32-row blocks
+// at the same columns - wave w takes row block w % 4 and, of each pair of wave-loads, number
+// w / 4 - so one 16*NB x 256 activation tile per stage serves all eight waves (read from L2 once
+// per 128 matrix rows instead of once per 32; the per-wave reads measured 35-50 % of the run
+// time before).  Tiles are double-buffered: loaded to registers two stages ahead, written to
+// LDS one stage ahead, one barrier per stage.  Rows of the tile are 512 bytes with the 16-byte
+// chunk index xor-ed with the row, which keeps both the 16-byte fills and the A-operand reads
+// (16 lanes = 16 rows at the same chunk) free of bank conflicts.
+// Work unit = (group of 4 row blocks, k split s); a workgroup keeps one s, so its sequence of
+// activation tiles is the same for every unit and the pipeline runs across unit boundaries.
+// S > 1 (few row blocks): fp32 partial results go to parts[s][batch][m] and are summed afterwards.
 constexpr int kGemmThreads = 512;  // 8 waves: up to 256 VGPRs for the accumulators
 constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kGemmRB = 4;          // row blocks per group
+constexpr size_t kGemmTileBytes = 32 * 512;  // 32 batch rows x 256 columns fp16
+constexpr size_t kGemmLds = kLut128Bytes + 2 * kGemmTileBytes;
 
 template <int K, int NB, int DEPTH>
 __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
-    float* __restrict__ out, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16) {
+    float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16, int S, int wl_per) {
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-  float* red = reinterpret_cast<float*>(smem + kLut128Bytes);  // [kGemmWaves][32][16*NB]
+  uint8_t* tiles = smem + kLut128Bytes;  // [2][16*NB rows][512 bytes]
+  constexpr uint32_t TILE = 16 * NB * 512;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rbi = wave & (kGemmRB - 1), ks = wave >> 2;
   const int a = lane & 15, g = lane >> 4;
   const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
   const int nkb = k >> 5;
-  const int nwl = (nkb + 3) >> 2;  // wave-loads per row block; a partial last one reads zeros for x
+  const int nwl = (nkb + 3) >> 2;  // wave-loads per row block; a partial last one meets zero activations
   const int nrb = m >> 5;
+  const int ngroups = (nrb + kGemmRB - 1) / kGemmRB;
   const uint32_t rb_bytes = (uint32_t)nkb * 128 * K;
   constexpr uint32_t WL_BYTES = 512 * K;
   const uint32_t loff = (uint32_t)lane * 8 * K;
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
-  constexpr int NC = 16 * NB;
 
-  // items of this wave: (row block, wave-load wave + 8*j), flat, DEPTH in flight
-  const int npw = (nwl + kGemmWaves - 1) / kGemmWaves;
-  const int nvj = wave < nwl ? (nwl - wave + kGemmWaves - 1) / kGemmWaves : 0;
-  const int upw = (nrb - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-  const int T = upw * npw;
-  int l_j = 0, l_t = 0;
-  uint32_t l_rboff = blockIdx.x * rb_bytes;
-  const uint32_t rb_step_bytes = gridDim.x * rb_bytes;
+  const int s = blockIdx.x % S;
+  const int g0 = blockIdx.x / S, gstep = gridDim.x / S;
+  const int wl0 = s * wl_per;                                   // wl_per is even
+  const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
+  const int nst = (wl1 - wl0 + 1) >> 1;                         // stages (pairs of wave-loads) per unit
+  const int upw = g0 < ngroups ? (ngroups - g0 + gstep - 1) / gstep : 0;  // units of this workgroup
+  const int T = upw * nst;
+  float* out_s = dst + (size_t)s * batch * m;
+
+  // ---- weight stream of this wave: item q = (unit q / nst, stage q % nst), DEPTH in flight
+  int l_t = 0, l_q = 0, l_grp = g0;
   LaneData<K> buf[DEPTH];
   auto issue = [&](int d) {
-    const bool valid = l_j < nvj && l_t < T;
-    const uint32_t wl = (uint32_t)(wave + l_j * kGemmWaves);
-    buf[d] = load_lane_buf<K>(rs_w, loff, valid ? l_rboff + wl * WL_BYTES : 0u);
-    ++l_t;
-    if (++l_j == npw) {
-      l_j = 0;
-      l_rboff += rb_step_bytes;
+    const int rb = l_grp * kGemmRB + rbi;
+    const int wl = wl0 + 2 * l_t + ks;
+    const bool valid = l_q < T && rb < nrb && wl < wl1;
+    buf[d] = load_lane_buf<K>(rs_w, loff, valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u);
+    ++l_q;
+    if (++l_t == nst) {
+      l_t = 0;
+      l_grp += gstep;
     }
   };
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(d);
-  build_lut128(lut, tlut, tid, kGemmThreads);
-  __syncthreads();
 
-  // activations: lane (batch row a of tile nb, K group g) reads x[b][128*wl + 32*g + 16*kh + 0..15]
-  // through a buffer descriptor that ends with the last batch row: the lanes of a ragged last
-  // wave-load (columns past k) and padding items get an offset past the end and read zeros,
-  // which cancel whatever those lanes decode.  The loads for item i+1 are issued before item i
-  // is decoded, so they have a whole stage to arrive.
-  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(x), 0, (int)((size_t)batch * k * 2), 0x00020000);
-  uint32_t xvoff[NB];
+  // ---- activation tiles: thread fills NB 16-byte chunks per tile
+  u32x4 xg[2][NB];  // tiles on their way: [parity of the stage][chunk]
+  auto load_tile = [&](int slot, int t) {  // stage t of a unit -> registers
+    const int col0 = 128 * (wl0 + 2 * t);
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int bb = 16 * nb + a;
-    xvoff[nb] = (uint32_t)(bb < batch ? bb : 0) * (uint32_t)k * 2u + 64u * g;
-  }
-  u32x4 xbuf[DEPTH][2][NB][2];  // [stage][kh][nb][low / high 16 bytes]
-  auto issue_x = [&](int d, int cj, bool item_ok) {
-    const int wl = wave + cj * kGemmWaves;
-    const bool ok = item_ok && cj < nvj && 128 * wl + 32 * g < k;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const uint32_t vo = ok ? xvoff[nb] : 0x7FFFFFC0u;
-#pragma unroll
-      for (int kh = 0; kh < 2; ++kh) {
-        xbuf[d][kh][nb][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, vo + 32u * kh, (uint32_t)wl * 256u, 0);
-        xbuf[d][kh][nb][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, vo + 32u * kh + 16u, (uint32_t)wl * 256u, 0);
-      }
+    for (int i = 0; i < NB; ++i) {
+      const int idx = i * kGemmThreads + tid;
+      const int b = idx >> 5, c = idx & 31;
+      const int col = col0 + 8 * c;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (b < batch && col < k && t < nst)
+        v = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + col);
+      xg[slot][i] = v;
     }
   };
-  issue_x(0, 0, T > 0);
+  auto store_tile = [&](int slot, int bufi) {  // registers -> LDS buffer
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int idx = i * kGemmThreads + tid;
+      const int b = idx >> 5, c = idx & 31;
+      *reinterpret_cast<u32x4*>(tiles + bufi * TILE + b * 512 + ((c ^ (b & 7)) << 4)) = xg[slot][i];
+    }
+  };
+  load_tile(0, 0);
+  load_tile(1, nst > 1 ? 1 : 0);
+  build_lut128(lut, tlut, tid, kGemmThreads);
+  store_tile(0, 0);
+  __syncthreads();
 
   float4_t acc[2][2][2][NB];  // [mh][rh][column half][batch tile]
 #pragma unroll
   for (int i = 0; i < 8 * NB; ++i) (&acc[0][0][0][0])[i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  int c_j = 0, c_rb = blockIdx.x;
-  for (int t = 0; t < T; t += DEPTH) {
+  // LDS byte offset (inside a tile) of this lane's A-operand chunks: row 16*nb + a, chunk 16*ks + 4*g + 2*kh + h
+  uint32_t arow[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) arow[nb] = (uint32_t)(16 * nb + a) * 512u;
+  const uint32_t a7 = (uint32_t)(a & 7);
+  const uint32_t tiles_addr = lds_address(tiles);
+
+  int c_t = 0, c_grp = g0;
+  for (int q = 0; q < T; q += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      issue_x((d + 1) % DEPTH, c_j + 1 == npw ? 0 : c_j + 1, t + d + 1 < T);
-      if (t + d < T && c_j < nvj) {
-        auto& xa = xbuf[d];
-        uint32_t P[16], W[32];
-        packed_states<K>(buf[d], P);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
-          W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
-          W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
+      const bool live = q + d < T;  // uniform over the workgroup
+      if (live) {
+        // tile of stage q+d+2 to registers (slot = parity of that stage = parity of q+d)
+        {
+          int t2 = c_t + 2;
+          if (t2 >= nst) t2 -= nst;
+          if (t2 >= nst) t2 -= nst;  // nst == 1
+          load_tile((q + d) & 1, t2);
         }
-        __builtin_amdgcn_sched_barrier(0);
+        const int rb = c_grp * kGemmRB + rbi;
+        const int wl = wl0 + 2 * c_t + ks;
+        if (rb < nrb && wl < wl1) {
+          typedef __attribute__((address_space(3))) const u32x4 lds_u32x4_t;
+          const uint32_t tb = tiles_addr + (uint32_t)((q + d) & 1) * TILE;
+          uint32_t P[16], W[32];
+          packed_states<K>(buf[d], P);
 #pragma unroll
-        for (int mh = 0; mh < 2; ++mh)
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t hq = pk_hash(P[i]) & 0xFFC0FFC0u;
+            W[2 * i] = lds_word_abs(lut128_addr_lo(hq, slot4));
+            W[2 * i + 1] = lds_word_abs(lut128_addr_hi(hq, slot4));
+          }
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int rh = 0; rh < 2; ++rh)
-#pragma unroll
-            for (int kh = 0; kh < 2; ++kh) {
-              const int tt = 2 * kh + mh;
-              const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
-                                W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
-              const half8_t bop = __builtin_bit_cast(half8_t, wv);
-#pragma unroll
-              for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int ch = 0; ch < 2; ++ch) {
-                  // columns +4*ch+{0..3} and +8+4*ch+{0..3} of the 16 loaded ones
-                  const u32x4 xv = {xa[kh][nb][0][2 * ch], xa[kh][nb][0][2 * ch + 1],
-                                    xa[kh][nb][1][2 * ch], xa[kh][nb][1][2 * ch + 1]};
-                  acc[mh][rh][ch][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                      __builtin_bit_cast(half8_t, xv), bop, acc[mh][rh][ch][nb], 0, 0, 0);
-                }
-            }
-      }
-      issue(d);
-      if (t + d < T && ++c_j == npw) {
-        // ---- end of a row block: pick the meaningful accumulator, add the
-        // partner lane, reduce across waves, store
-#pragma unroll
-        for (int mh = 0; mh < 2; ++mh)
-#pragma unroll
-          for (int rh = 0; rh < 2; ++rh)
+          for (int kh = 0; kh < 2; ++kh) {
+            u32x4 xa[NB][2];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                float v = (a & 1) ? acc[mh][rh][1][nb][i] : acc[mh][rh][0][nb][i];
-                v += dpp_xor1(v);
-                acc[mh][rh][0][nb][i] = 0.f;
-                acc[mh][rh][1][nb][i] = 0.f;
-                // lane (g, a even): batch row 16*nb + 4*g + i, matrix row 16*mh + 8*rh + a/2
-                if ((a & 1) == 0)
-                  red[(wave * 32 + 16 * mh + 8 * rh + (a >> 1)) * NC + 16 * nb + 4 * g + i] = v;
+              for (int h = 0; h < 2; ++h) {
+                const uint32_t c = (uint32_t)(16 * ks + 4 * g + 2 * kh + h) ^ a7;
+                xa[nb][h] = *(lds_u32x4_t*)(uintptr_t)(tb + arow[nb] + (c << 4));
               }
-        __syncthreads();
-        for (int e = tid; e < 32 * NC; e += kGemmThreads) {
-          const int bb = e >> 5, row = e & 31;  // consecutive threads -> consecutive rows of out
-          float sum = 0.f;
 #pragma unroll
-          for (int w = 0; w < kGemmWaves; ++w) sum += red[(w * 32 + row) * NC + bb];
-          if (round_f16) sum = (float)(_Float16)sum;
-          if (bb < batch) out[(size_t)bb * m + c_rb * 32 + row] = sum;
+            for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+              for (int rh = 0; rh < 2; ++rh) {
+                const int tt = 2 * kh + mh;
+                const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
+                                  W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
+                const half8_t bop = __builtin_bit_cast(half8_t, wv);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                  for (int ch = 0; ch < 2; ++ch) {
+                    // columns +4*ch+{0..3} and +8+4*ch+{0..3} of the 16 loaded ones
+                    const u32x4 xv = {xa[nb][0][2 * ch], xa[nb][0][2 * ch + 1], xa[nb][1][2 * ch],
+                                      xa[nb][1][2 * ch + 1]};
+                    acc[mh][rh][ch][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8_t, xv), bop, acc[mh][rh][ch][nb], 0, 0, 0);
+                  }
+              }
+          }
         }
+      }
+      issue(d);
+      if (live) {
+        // tile of the next stage (in registers since the previous stage) into the other buffer
+        store_tile((q + d + 1) & 1, (q + d + 1) & 1);
         __syncthreads();
-        c_j = 0;
-        c_rb += gridDim.x;
+        if (++c_t == nst) {
+          // ---- end of a unit: the two k halves of a row block meet in the buffer this stage used
+          // (the next tile sits in the other one), the wave of half 0 adds, rounds and stores
+          float* xch = reinterpret_cast<float*>(tiles + ((q + d) & 1) * TILE) + rbi * (16 * NB * 32);
+          float vals[2][2][NB][4];
+#pragma unroll
+          for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+            for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+              for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                  float v = (a & 1) ? acc[mh][rh][1][nb][i] : acc[mh][rh][0][nb][i];
+                  v += dpp_xor1(v);
+                  vals[mh][rh][nb][i] = v;
+                  acc[mh][rh][0][nb][i] = 0.f;
+                  acc[mh][rh][1][nb][i] = 0.f;
+                }
+          const int e0 = ((a >> 1) + 8 * g) * (16 * NB);  // even lanes: 32 slots of 16*NB floats
+          if (ks == 1 && (a & 1) == 0) {
+#pragma unroll
+            for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+              for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                  *reinterpret_cast<float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4) =
+                      float4_t{vals[mh][rh][nb][0], vals[mh][rh][nb][1], vals[mh][rh][nb][2], vals[mh][rh][nb][3]};
+          }
+          __syncthreads();
+          const int rb = c_grp * kGemmRB + rbi;
+          if (ks == 0 && (a & 1) == 0 && rb < nrb) {
+#pragma unroll
+            for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+              for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                  const float4_t o = *reinterpret_cast<const float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4);
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) {
+                    float sum = vals[mh][rh][nb][i] + o[i];
+                    if (round_f16) sum = (float)(_Float16)sum;
+                    // lane (g, a even): batch row 16*nb + 4*g + i, matrix row 16*mh + 8*rh + a/2
+                    const int bb = 16 * nb + 4 * g + i;
+                    if (bb < batch) out_s[(size_t)bb * m + rb * 32 + 16 * mh + 8 * rh + (a >> 1)] = sum;
+                  }
+                }
+          }
+          __syncthreads();  // the exchange buffer becomes a tile again at the end of the next stage
+          c_t = 0;
+          c_grp += gstep;
+        }
       }
     }
   }
+}
+
+// out[i] = parts[0][i] + ... (+ rounding through fp16) for the split-k GEMM
+__global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict__ out,
+                                                              const float* __restrict__ parts, long n,
+                                                              int S, int round_f16) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float sum = parts[i];
+  for (int s = 1; s < S; ++s) sum += parts[(size_t)s * n + i];
+  out[i] = round_f16 ? (float)(_Float16)sum : sum;
 }
 
 // ---------------------------------------------------------------------------
@@ -554,7 +639,6 @@ hipError_t allow_lds(F* fn, size_t bytes) {
                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-constexpr size_t kGemmLds = kLut128Bytes + (size_t)kGemmWaves * 32 * 32 * sizeof(float);
 
 hipError_t setup_once() {
   static hipError_t status = [] {
@@ -624,7 +708,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 4; }
+int qtip_abi_version(void) { return 5; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -747,8 +831,27 @@ int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, co
   return (int)hipGetLastError();
 }
 
+// k split of the batched GEMM: groups of 4 row blocks are the parallel units, so matrices with
+// few rows are also cut along k (only when the caller provides room for the partial results)
+static int gemm_split(int m, int k, int cus) {
+  const int ngroups = ((m >> 5) + kGemmRB - 1) / kGemmRB;
+  const int nwl = ((k >> 5) + 3) >> 2;
+  int S = 1;
+  while (S < kMaxSplit && ngroups * S * 2 <= cus && nwl / (S * 2) >= 8) S *= 2;
+  return S;
+}
+
+size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch) {
+  if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4 || batch < 1) return 0;
+  DeviceInfo& di = device_info();
+  if (!di.ok) return 0;
+  const int S = gemm_split(m, k, di.cus);
+  return S > 1 ? (size_t)S * (batch < 32 ? batch : 32) * m * sizeof(float) : 0;
+}
+
 int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, const void* tlut,
-                         int m, int k, int bits, int batch, int round_f16, void* stream) {
+                         int m, int k, int bits, int batch, int round_f16, void* workspace,
+                         size_t workspace_bytes, void* stream) {
   int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (batch < 1 || batch > 65535) return QTIP_E_SHAPE;
@@ -759,8 +862,21 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   if (!di.ok) return (int)hipErrorInvalidDevice;
   hipError_t e = setup_once();
   if (e != hipSuccess) return (int)e;
-  const int nrb = m >> 5;
-  const int grid = nrb < di.cus ? nrb : di.cus;
+  int S = 1;
+  if (workspace) {
+    S = gemm_split(m, k, di.cus);
+    if (S > 1 && workspace_bytes < (size_t)S * (batch < 32 ? batch : 32) * m * sizeof(float))
+      return QTIP_E_WORKSPACE;
+    if (!aligned16(workspace)) return QTIP_E_ALIGN;
+  }
+  const int ngroups = ((m >> 5) + kGemmRB - 1) / kGemmRB;
+  const int nwl = ((k >> 5) + 3) >> 2;
+  int wl_per = (nwl + S - 1) / S;
+  wl_per += wl_per & 1;              // stages are pairs of wave-loads
+  S = (nwl + wl_per - 1) / wl_per;   // rounding up may have emptied the last ranges
+  const long units = (long)ngroups * S;
+  long grid = units < di.cus ? units : di.cus;
+  grid -= grid % S;  // a workgroup keeps one k range
   hipStream_t st = (hipStream_t)stream;
   auto* p = (const uint8_t*)packed;
   auto* t = (const uint32_t*)tlut;
@@ -768,9 +884,12 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   for (int b0 = 0; b0 < batch; b0 += 32) {
     const int nb = batch - b0 < 32 ? batch - b0 : 32;
     float* o = out + (size_t)b0 * m;
+    float* d = S > 1 ? (float*)workspace : o;
+    const int rnd = S > 1 ? 0 : round_f16;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
-#define QTIP_GEMM(KB, NBT) \
-  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2)><<<grid, kGemmThreads, kGemmLds, st>>>(o, p, xx, t, m, k, nb, round_f16)
+#define QTIP_GEMM(KB, NBT)                                                                        \
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2)><<<(int)grid, kGemmThreads, kGemmLds, st>>>( \
+      d, p, xx, t, m, k, nb, rnd, S, wl_per)
 #define QTIP_GEMM_K(KB)            \
   if (nb <= 16) QTIP_GEMM(KB, 1);  \
   else QTIP_GEMM(KB, 2);
@@ -783,6 +902,12 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
 #undef QTIP_GEMM
     hipError_t le = hipGetLastError();
     if (le != hipSuccess) return (int)le;
+    if (S > 1) {
+      const long n = (long)nb * m;
+      sum_parts_round_kernel<<<(int)((n + 255) / 256), 256, 0, st>>>(o, (const float*)workspace, n, S, round_f16);
+      le = hipGetLastError();
+      if (le != hipSuccess) return (int)le;
+    }
   }
   return QTIP_OK;
 }

@@ -128,9 +128,17 @@ def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     out = torch.empty((batch, m), dtype=torch.float32, device=packed.device)
     if batch == 0:
         return out
+    L = lib()
     with torch.cuda.device(packed.device):
-        check(lib().qtip_decompress_gemm(_ptr(out), _ptr(packed), _ptr(x), _ptr(tlut), m, k, bits, batch,
-                                         int(bool(round_f16)), stream_ptr(packed.device)), "qtip_decompress_gemm")
+        need = L.qtip_gemm_workspace_bytes(m, k, bits, batch)
+        if need:
+            ws = _workspace(packed.device, need)
+            wsp, wsb = _ptr(ws), ws.numel()
+        else:
+            wsp, wsb = ctypes.c_void_p(0), 0
+        check(L.qtip_decompress_gemm(_ptr(out), _ptr(packed), _ptr(x), _ptr(tlut), m, k, bits, batch,
+                                     int(bool(round_f16)), wsp, wsb, stream_ptr(packed.device)),
+              "qtip_decompress_gemm")
     return out
 
 

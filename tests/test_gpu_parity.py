@@ -137,6 +137,31 @@ def test_gemm_vs_oracle(K, shape, batch):
     assert np.array_equal(got16, got.astype(np.float16).astype(np.float32))
 
 
+@pytest.mark.parametrize("K", [2, 4])
+@pytest.mark.parametrize("shape", [(128, 4096), (96, 8192 + 64), (160, 2048 + 32), (4096 + 32, 512)])
+@pytest.mark.parametrize("batch", [5, 32, 40])
+def test_gemm_split_k_and_ragged_groups(K, shape, batch):
+    """Few row blocks: k is cut (partials through the workspace, extra summing launch); row-block
+    counts that are not a multiple of 4 leave waves of the last group without work."""
+    from qtip_amd import ops
+    from qtip_amd._lib import lib
+    m, k = shape
+    if m <= 160 and k >= 4096:
+        assert lib().qtip_gemm_workspace_bytes(m, k, K, batch) > 0
+    L = make_layer(m, k, K, seed=m + k + K + batch)
+    rng = np.random.default_rng(batch)
+    X = rng.standard_normal((batch, k)).astype(np.float16)
+    pk, xd, tl = dev(L["packed"]), dev(X), dev(L["tlut"])
+    ops._workspace(pk.device, 1).fill_(0xFF)  # NaN patterns: a partial result that is never written shows
+    got = ops.decompress_gemm(pk, xd, tl, m, k, K, round_f16=False).cpu().numpy()
+    w = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float64)
+    assert_close(got, X.astype(np.float64) @ w.T)
+    again = ops.decompress_gemm(pk, xd, tl, m, k, K, round_f16=False).cpu().numpy()
+    assert np.array_equal(got, again)  # deterministic
+    got16 = ops.decompress_gemm(pk, xd, tl, m, k, K, round_f16=True).cpu().numpy()
+    assert np.array_equal(got16, got.astype(np.float16).astype(np.float32))
+
+
 @pytest.mark.parametrize("n", [2, 16, 64, 128, 256, 1024, 4096, 8192, 32768, 131072])
 @pytest.mark.parametrize("rows", [1, 3])
 def test_rht_pow2(n, rows):

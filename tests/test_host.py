@@ -40,7 +40,8 @@ def test_argument_rejection_without_gpu():
     assert L.qtip_decompress_matvec(p, p, p, p, 64, 64, 5, null, 0, null) == -1
     assert L.qtip_decompress_matvec(null, p, p, p, 64, 64, 2, null, 0, null) == -2
     assert L.qtip_decode(p, p, null, 64, 64, 2, null) == -2
-    assert L.qtip_decompress_gemm(p, p, p, p, 64, 64, 2, 0, 0, null) == -1
+    assert L.qtip_decompress_gemm(p, p, p, p, 64, 64, 2, 0, 0, null, 0, null) == -1
+    assert L.qtip_gemm_workspace_bytes(33, 64, 2, 8) == 0
     assert L.qtip_rht(p, 0, p, 0, 1, 1, 100, 1, null, null, null, 1.0, null) == -1  # not a power of two
     assert L.qtip_rht(p, 0, p, 0, 1, 1, 12 * 64, 12, null, null, null, 1.0, null) == -2  # table missing
     assert L.qtip_rht(p, 7, p, 0, 1, 1, 64, 1, null, null, null, 1.0, null) == -5
