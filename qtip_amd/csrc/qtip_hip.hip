@@ -379,20 +379,26 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(float* __restrict__ out,
 // Work unit = (group of 4 row blocks, k split s); a workgroup keeps one s, so its sequence of
 // activation tiles is the same for every unit and the pipeline runs across unit boundaries.
 // S > 1 (few row blocks): fp32 partial results go to parts[s][batch][m] and are summed afterwards.
-constexpr int kGemmThreads = 512;  // 8 waves: up to 256 VGPRs for the accumulators
-constexpr int kGemmWaves = kGemmThreads / 64;
-constexpr int kGemmRB = 4;          // row blocks per group
-constexpr size_t kGemmTileBytes = 32 * 512;  // 32 batch rows x 256 columns fp16
+constexpr int kGemmRB = 4;  // row blocks per group
+// Two shapes of workgroup: 8 waves (2 k slices, up to 256 VGPRs: two batch tiles) and 16 waves
+// (4 k slices, 128 VGPRs: one batch tile, twice the waves to hide the latencies of a stage).
+constexpr size_t kGemmTileBytes = 16 * 1024;  // 16*NB batch rows x 256*KS columns fp16, NB*KS == 4
 constexpr size_t kGemmLds = kLut128Bytes + 2 * kGemmTileBytes;
 
-template <int K, int NB, int DEPTH>
-__global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
+template <int K, int NB, int DEPTH, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
     const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16, int S, int wl_per) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int KS = WAVES / kGemmRB;          // wave-loads per stage
+  constexpr int ROWB = KS * 256;               // bytes per tile row
+  constexpr int CPR = ROWB / 16;               // 16-byte chunks per tile row
+  constexpr uint32_t TILE = 16 * NB * ROWB;
+  static_assert(2 * TILE <= 2 * kGemmTileBytes, "tiles do not fit");
+  static_assert(16 * NB * CPR == NB * THREADS, "NB chunks per thread and tile");
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-  uint8_t* tiles = smem + kLut128Bytes;  // [2][16*NB rows][512 bytes]
-  constexpr uint32_t TILE = 16 * NB * 512;
+  uint8_t* tiles = smem + kLut128Bytes;  // [2][16*NB rows][ROWB bytes]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rbi = wave & (kGemmRB - 1), ks = wave >> 2;
@@ -410,9 +416,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 
   const int s = blockIdx.x % S;
   const int g0 = blockIdx.x / S, gstep = gridDim.x / S;
-  const int wl0 = s * wl_per;                                   // wl_per is even
+  const int wl0 = s * wl_per;                                   // wl_per is a multiple of KS
   const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
-  const int nst = (wl1 - wl0 + 1) >> 1;                         // stages (pairs of wave-loads) per unit
+  const int nst = wl1 > wl0 ? (wl1 - wl0 + KS - 1) / KS : 0;    // stages (KS wave-loads each) per unit
   const int upw = g0 < ngroups ? (ngroups - g0 + gstep - 1) / gstep : 0;  // units of this workgroup
   const int T = upw * nst;
   float* out_s = dst + (size_t)s * batch * m;
@@ -422,7 +428,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
   LaneData<K> buf[DEPTH];
   auto issue = [&](int d) {
     const int rb = l_grp * kGemmRB + rbi;
-    const int wl = wl0 + 2 * l_t + ks;
+    const int wl = wl0 + KS * l_t + ks;
     const bool valid = l_q < T && rb < nrb && wl < wl1;
     buf[d] = load_lane_buf<K>(rs_w, loff, valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u);
     ++l_q;
@@ -437,29 +443,28 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
   // ---- activation tiles: thread fills NB 16-byte chunks per tile
   u32x4 xg[2][NB];  // tiles on their way: [parity of the stage][chunk]
   auto load_tile = [&](int slot, int t) {  // stage t of a unit -> registers
-    const int col0 = 128 * (wl0 + 2 * t);
+    const int col0 = 128 * (wl0 + KS * t);
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int idx = i * kGemmThreads + tid;
-      const int b = idx >> 5, c = idx & 31;
+      const int idx = i * THREADS + tid;
+      const int b = idx / CPR, c = idx % CPR;
       const int col = col0 + 8 * c;
       u32x4 v = {0u, 0u, 0u, 0u};
-      if (b < batch && col < k && t < nst)
-        v = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + col);
+      if (b < batch && col < k) v = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + col);
       xg[slot][i] = v;
     }
   };
   auto store_tile = [&](int slot, int bufi) {  // registers -> LDS buffer
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      const int idx = i * kGemmThreads + tid;
-      const int b = idx >> 5, c = idx & 31;
-      *reinterpret_cast<u32x4*>(tiles + bufi * TILE + b * 512 + ((c ^ (b & 7)) << 4)) = xg[slot][i];
+      const int idx = i * THREADS + tid;
+      const int b = idx / CPR, c = idx % CPR;
+      *reinterpret_cast<u32x4*>(tiles + bufi * TILE + b * ROWB + ((c ^ (b & 7)) << 4)) = xg[slot][i];
     }
   };
   load_tile(0, 0);
   load_tile(1, nst > 1 ? 1 : 0);
-  build_lut128(lut, tlut, tid, kGemmThreads);
+  build_lut128(lut, tlut, tid, THREADS);
   store_tile(0, 0);
   __syncthreads();
 
@@ -470,7 +475,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
   // LDS byte offset (inside a tile) of this lane's A-operand chunks: row 16*nb + a, chunk 16*ks + 4*g + 2*kh + h
   uint32_t arow[NB];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) arow[nb] = (uint32_t)(16 * nb + a) * 512u;
+  for (int nb = 0; nb < NB; ++nb) arow[nb] = (uint32_t)(16 * nb + a) * ROWB;
   const uint32_t a7 = (uint32_t)(a & 7);
   const uint32_t tiles_addr = lds_address(tiles);
 
@@ -488,7 +493,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
           load_tile((q + d) & 1, t2);
         }
         const int rb = c_grp * kGemmRB + rbi;
-        const int wl = wl0 + 2 * c_t + ks;
+        const int wl = wl0 + KS * c_t + ks;
         if (rb < nrb && wl < wl1) {
           typedef __attribute__((address_space(3))) const u32x4 lds_u32x4_t;
           const uint32_t tb = tiles_addr + (uint32_t)((q + d) & 1) * TILE;
@@ -539,8 +544,9 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
         store_tile((q + d + 1) & 1, (q + d + 1) & 1);
         __syncthreads();
         if (++c_t == nst) {
-          // ---- end of a unit: the two k halves of a row block meet in the buffer this stage used
-          // (the next tile sits in the other one), the wave of half 0 adds, rounds and stores
+          // ---- end of a unit: the k slices of a row block meet in the buffer this stage used
+          // (the next tile sits in the other one): slices 1 .. KS-1 hand their sums over in turn,
+          // the wave of slice 0 adds them in that order, rounds and stores
           float* xch = reinterpret_cast<float*>(tiles + ((q + d) & 1) * TILE) + rbi * (16 * NB * 32);
           float vals[2][2][NB][4];
 #pragma unroll
@@ -558,17 +564,32 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
                   acc[mh][rh][1][nb][i] = 0.f;
                 }
           const int e0 = ((a >> 1) + 8 * g) * (16 * NB);  // even lanes: 32 slots of 16*NB floats
-          if (ks == 1 && (a & 1) == 0) {
+          for (int turn = 1; turn < KS; ++turn) {
+            if (ks == turn && (a & 1) == 0) {
 #pragma unroll
-            for (int mh = 0; mh < 2; ++mh)
+              for (int mh = 0; mh < 2; ++mh)
 #pragma unroll
-              for (int rh = 0; rh < 2; ++rh)
+                for (int rh = 0; rh < 2; ++rh)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                  *reinterpret_cast<float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4) =
-                      float4_t{vals[mh][rh][nb][0], vals[mh][rh][nb][1], vals[mh][rh][nb][2], vals[mh][rh][nb][3]};
+                  for (int nb = 0; nb < NB; ++nb)
+                    *reinterpret_cast<float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4) =
+                        float4_t{vals[mh][rh][nb][0], vals[mh][rh][nb][1], vals[mh][rh][nb][2], vals[mh][rh][nb][3]};
+            }
+            __syncthreads();
+            if (ks == 0 && (a & 1) == 0) {
+#pragma unroll
+              for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+                for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+                  for (int nb = 0; nb < NB; ++nb) {
+                    const float4_t o = *reinterpret_cast<const float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vals[mh][rh][nb][i] += o[i];
+                  }
+            }
+            __syncthreads();  // the next slice may overwrite; after the last turn the buffer becomes a tile again
           }
-          __syncthreads();
           const int rb = c_grp * kGemmRB + rbi;
           if (ks == 0 && (a & 1) == 0 && rb < nrb) {
 #pragma unroll
@@ -576,19 +597,16 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gemm_kernel(
 #pragma unroll
               for (int rh = 0; rh < 2; ++rh)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                  const float4_t o = *reinterpret_cast<const float4_t*>(xch + e0 + ((mh * 2 + rh) * NB + nb) * 4);
+                for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                   for (int i = 0; i < 4; ++i) {
-                    float sum = vals[mh][rh][nb][i] + o[i];
+                    float sum = vals[mh][rh][nb][i];
                     if (round_f16) sum = (float)(_Float16)sum;
                     // lane (g, a even): batch row 16*nb + 4*g + i, matrix row 16*mh + 8*rh + a/2
                     const int bb = 16 * nb + 4 * g + i;
                     if (bb < batch) out_s[(size_t)bb * m + rb * 32 + 16 * mh + 8 * rh + (a >> 1)] = sum;
                   }
-                }
           }
-          __syncthreads();  // the exchange buffer becomes a tile again at the end of the next stage
           c_t = 0;
           c_grp += gstep;
         }
@@ -654,12 +672,12 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, kD2X, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((gemm_kernel<2, 1, 4>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<2, 2, 4>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 1, 3>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 2, 3>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 1, 2>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 2, 2>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 1, 3, 16>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 2, 3, 8>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
 #undef QTIP_ALLOW
     return hipSuccess;
   }();
@@ -871,28 +889,31 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   }
   const int ngroups = ((m >> 5) + kGemmRB - 1) / kGemmRB;
   const int nwl = ((k >> 5) + 3) >> 2;
-  int wl_per = (nwl + S - 1) / S;
-  wl_per += wl_per & 1;              // stages are pairs of wave-loads
-  S = (nwl + wl_per - 1) / wl_per;   // rounding up may have emptied the last ranges
-  const long units = (long)ngroups * S;
-  long grid = units < di.cus ? units : di.cus;
-  grid -= grid % S;  // a workgroup keeps one k range
   hipStream_t st = (hipStream_t)stream;
   auto* p = (const uint8_t*)packed;
   auto* t = (const uint32_t*)tlut;
-  // batch handled in passes of at most 32 rows (two 16-row MFMA tiles)
+  // batch handled in passes of at most 32 rows: two 16-row MFMA tiles on the 8-wave workgroup;
+  // up to 16 rows run on the 16-wave workgroup (4 wave-loads per stage)
   for (int b0 = 0; b0 < batch; b0 += 32) {
     const int nb = batch - b0 < 32 ? batch - b0 : 32;
+    const int KS = nb <= 16 ? 4 : 2;
+    int Sp = S;
+    int wl_per = (nwl + Sp - 1) / Sp;
+    wl_per = (wl_per + KS - 1) / KS * KS;  // stages are groups of KS wave-loads
+    Sp = (nwl + wl_per - 1) / wl_per;      // rounding up may have emptied the last ranges
+    const long units = (long)ngroups * Sp;
+    long grid = units < di.cus ? units : di.cus;
+    grid -= grid % Sp;  // a workgroup keeps one k range
     float* o = out + (size_t)b0 * m;
-    float* d = S > 1 ? (float*)workspace : o;
-    const int rnd = S > 1 ? 0 : round_f16;
+    float* d = Sp > 1 ? (float*)workspace : o;
+    const int rnd = Sp > 1 ? 0 : round_f16;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
-#define QTIP_GEMM(KB, NBT)                                                                        \
-  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2)><<<(int)grid, kGemmThreads, kGemmLds, st>>>( \
-      d, p, xx, t, m, k, nb, rnd, S, wl_per)
-#define QTIP_GEMM_K(KB)            \
-  if (nb <= 16) QTIP_GEMM(KB, 1);  \
-  else QTIP_GEMM(KB, 2);
+#define QTIP_GEMM(KB, NBT, WV)                                                                          \
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2), WV><<<(int)grid, WV * 64, kGemmLds, st>>>(      \
+      d, p, xx, t, m, k, nb, rnd, Sp, wl_per)
+#define QTIP_GEMM_K(KB)               \
+  if (nb <= 16) QTIP_GEMM(KB, 1, 16); \
+  else QTIP_GEMM(KB, 2, 8);
     switch (bits) {
       case 2: QTIP_GEMM_K(2) break;
       case 3: QTIP_GEMM_K(3) break;
@@ -902,9 +923,9 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
 #undef QTIP_GEMM
     hipError_t le = hipGetLastError();
     if (le != hipSuccess) return (int)le;
-    if (S > 1) {
+    if (Sp > 1) {
       const long n = (long)nb * m;
-      sum_parts_round_kernel<<<(int)((n + 255) / 256), 256, 0, st>>>(o, (const float*)workspace, n, S, round_f16);
+      sum_parts_round_kernel<<<(int)((n + 255) / 256), 256, 0, st>>>(o, (const float*)workspace, n, Sp, round_f16);
       le = hipGetLastError();
       if (le != hipSuccess) return (int)le;
     }
