@@ -27,10 +27,11 @@ __device__ __forceinline__ float wave_reduce_sum(float v) {
 // One workgroup per query head.  qkv: [H*D | Hkv*D | Hkv*D] fp16 of the new
 // token; k_cache / v_cache: [Hkv][max_len][D] fp16; pos_ptr: position of the
 // new token (device memory, so that a recorded graph follows the position).
+template <int D>
 __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     _Float16* __restrict__ out, const _Float16* __restrict__ qkv, _Float16* __restrict__ k_cache,
     _Float16* __restrict__ v_cache, const long* __restrict__ pos_ptr,
-    const float* __restrict__ inv_freq, int H, int Hkv, int D, int max_len) {
+    const float* __restrict__ inv_freq, int H, int Hkv, int max_len) {
   extern __shared__ __align__(16) uint8_t smem[];
   float* q_s = reinterpret_cast<float*>(smem);   // [D] rotated query (as fp16 values)
   float* k_s = q_s + kMaxHeadDim;                // [D] rotated new key
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int h = blockIdx.x, rep = H / Hkv, kvh = h / rep;
   const int pos = (int)pos_ptr[0];
-  const int half = D >> 1;
+  constexpr int half = D >> 1;
   const _Float16* q_in = qkv + (size_t)h * D;
   const _Float16* k_in = qkv + (size_t)H * D + (size_t)kvh * D;
   const _Float16* v_in = qkv + (size_t)(H + Hkv) * D + (size_t)kvh * D;
@@ -72,31 +73,42 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   const float sm_scale = rsqrtf((float)D);
   const int nkeys = pos + 1 < max_len ? pos + 1 : max_len;
   const int sub = tid & 7, kq = tid >> 3;
-  const int dper = D >> 3;  // dims per lane (multiple of 8: D % 64 == 0)
+  constexpr int dper = D >> 3;  // dims per lane (multiple of 8: D % 64 == 0)
   float mx = -INFINITY;
-  for (int t0 = 0; t0 < nkeys; t0 += kAttnThreads / 8) {
-    const int t = t0 + kq;
-    float s = 0.f;
-    if (t < nkeys) {
+  // four keys per thread group and round, all of their loads issued before the first use
+  constexpr int KU = 4;
+  for (int t0 = 0; t0 < nkeys; t0 += KU * (kAttnThreads / 8)) {
+    uint4 raw[KU][dper / 8];
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int t = t0 + kq + u * (kAttnThreads / 8);
+      const int tc = (t < nkeys && t != pos) ? t : 0;  // clamped: the new key comes from LDS
+      const uint4* kr = reinterpret_cast<const uint4*>(kc + (size_t)tc * D + sub * dper);
+#pragma unroll
+      for (int d8 = 0; d8 < dper / 8; ++d8) raw[u][d8] = kr[d8];
+    }
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int t = t0 + kq + u * (kAttnThreads / 8);
+      float s = 0.f;
       if (t == pos) {
         for (int d = 0; d < dper; ++d) s += q_s[sub * dper + d] * k_s[sub * dper + d];
       } else {
-        const uint4* kr = reinterpret_cast<const uint4*>(kc + (size_t)t * D + sub * dper);
+#pragma unroll
         for (int d8 = 0; d8 < dper / 8; ++d8) {
-          const uint4 raw = kr[d8];
-          const _Float16* hv = reinterpret_cast<const _Float16*>(&raw);
+          const _Float16* hv = reinterpret_cast<const _Float16*>(&raw[u][d8]);
 #pragma unroll
           for (int e = 0; e < 8; ++e) s += q_s[sub * dper + d8 * 8 + e] * (float)hv[e];
         }
       }
-    }
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2);
-    s += __shfl_xor(s, 4);
-    s *= sm_scale;
-    if (t < nkeys) {
-      if (sub == 0) p_s[t] = s;
-      mx = fmaxf(mx, s);
+      s += __shfl_xor(s, 1);
+      s += __shfl_xor(s, 2);
+      s += __shfl_xor(s, 4);
+      s *= sm_scale;
+      if (t < nkeys) {
+        if (sub == 0) p_s[t] = s;
+        mx = fmaxf(mx, s);
+      }
     }
   }
   mx = wave_reduce_max(mx);
@@ -121,28 +133,52 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   const float inv = 1.f / tot;
 
   // ---- output: thread (tg, dg) sums keys tg, tg+TG, ... for dims 8*dg .. 8*dg+7
-  const int DG = D >> 3, TG = kAttnThreads / DG;  // 16 dim groups, 64 key groups for D = 128
+  constexpr int DG = D >> 3, TG = kAttnThreads / DG;  // 16 dim groups, 64 key groups for D = 128
   const int dg = tid % DG, tg = tid / DG;
   float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int t = tg; t < nkeys; t += TG) {
-    const float pt = p_s[t];
-    if (t == pos) {
+  constexpr int VU = 8;  // values per thread and round, loaded before the first use
+  for (int t0 = tg; t0 < nkeys; t0 += VU * TG) {
+    uint4 raw[VU];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] += pt * v_s[dg * 8 + e];
-    } else {
-      const uint4 raw = *reinterpret_cast<const uint4*>(vc + (size_t)t * D + dg * 8);
-      const _Float16* hv = reinterpret_cast<const _Float16*>(&raw);
+    for (int u = 0; u < VU; ++u) {
+      const int t = t0 + u * TG;
+      const int tc = (t < nkeys && t != pos) ? t : 0;
+      raw[u] = *reinterpret_cast<const uint4*>(vc + (size_t)tc * D + dg * 8);
+    }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] += pt * (float)hv[e];
+    for (int u = 0; u < VU; ++u) {
+      const int t = t0 + u * TG;
+      if (t < nkeys) {
+        const float pt = p_s[t];
+        if (t == pos) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] += pt * v_s[dg * 8 + e];
+        } else {
+          const _Float16* hv = reinterpret_cast<const _Float16*>(&raw[u]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] += pt * (float)hv[e];
+        }
+      }
     }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[tg * D + dg * 8 + e] = o[e];
   __syncthreads();
-  // tree over the TG partial rows
-  for (int half_n = TG >> 1; half_n >= 1; half_n >>= 1) {
-    for (int i = tid; i < half_n * D; i += kAttnThreads) acc[i] += acc[i + half_n * D];
+  // two-level sum over the TG partial rows: thread (part, d) adds TG/PARTS rows, then PARTS rows
+  {
+    constexpr int PARTS = kAttnThreads / D;  // 8 for D = 128 (TG = 64 rows)
+    const int d = tid % D, part = tid / D;
+    constexpr int per = TG / PARTS;
+    float sum = 0.f;
+    for (int r = 0; r < per; ++r) sum += acc[(part * per + r) * D + d];
     __syncthreads();
+    acc[part * D + d] = sum;
+    __syncthreads();
+    if (tid < D) {
+      float tot2 = 0.f;
+      for (int r = 0; r < PARTS; ++r) tot2 += acc[r * D + tid];
+      acc[tid] = tot2;  // only read by this thread below
+    }
   }
   if (tid < D) out[(size_t)h * D + tid] = (_Float16)(acc[tid] * inv);
 }
@@ -157,8 +193,15 @@ extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k
       (head_dim & (head_dim - 1)) || max_len < 1 || max_len > 4096)
     return QTIP_E_SHAPE;
   const size_t lds = (size_t)(3 * kMaxHeadDim + 32 + 8192 + max_len) * sizeof(float);
-  decode_attn_kernel<<<heads, kAttnThreads, lds, (hipStream_t)stream>>>(
-      (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,
-      (const long*)pos_i64, inv_freq, heads, kv_heads, head_dim, max_len);
+#define QTIP_ATTN(DD)                                                                               \
+  decode_attn_kernel<DD><<<heads, kAttnThreads, lds, (hipStream_t)stream>>>(                          \
+      (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,  \
+      (const long*)pos_i64, inv_freq, heads, kv_heads, max_len)
+  switch (head_dim) {
+    case 64: QTIP_ATTN(64); break;
+    case 128: QTIP_ATTN(128); break;
+    default: QTIP_ATTN(256); break;
+  }
+#undef QTIP_ATTN
   return (int)hipGetLastError();
 }
