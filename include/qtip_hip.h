@@ -140,6 +140,19 @@ int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int i
                    int pre_mode, const void* norm_weight_f16, float eps,
                    const void* residual_f16, void* stream);
 
+/* Output transform of one linear layer, residual addition, RMSNorm and the input transform of the
+ * next linear layer for one hidden-size vector per row, in one launch (one workgroup per row):
+ *   x_out  = fp16(residual + fp16(post * scale_out * H_n (sum over in_parts of parts)))
+ *   xt_out = fp16(scale_in * H_n (pre * fp16(w * fp16(x_out * rsqrt(mean(x_out^2) + eps)))))
+ * i.e. qtip_rht_fused(residual) followed by qtip_rht_fused(pre_mode 1) (model/llama.py:129-135,
+ * 964-979 between two BitshiftLinear.forward calls, lib/codebook/bitshift.py:428-472).
+ * n in {2048, 4096, 8192} (both transforms of order 1); parts is [in_parts][rows][n] fp32,
+ * post fp32[n] or NULL, pre fp16[n] or NULL, residual / x_out / xt_out fp16 [rows][n]. */
+int qtip_rht_chain(void* xt_out_f16, void* x_out_f16, const float* parts, int in_parts, int rows, int n,
+                   const float* post_f32, float scale_out, const void* residual_f16,
+                   const void* norm_weight_f16, float eps, const void* pre_f16, float scale_in,
+                   void* stream);
+
 /* Single-token decode attention for the end-to-end loop, one launch: rotary embedding of q and
  * k in fp16 arithmetic (model/llama.py:264-295), write of k and v into the static cache at the
  * token's position (model/cache_utils.py:1173-1193), softmax(q K^T / sqrt(d)) V over cache slots

@@ -580,6 +580,151 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
   return launch_rht_l<float, float, false>(P, grid, loads, ri, st);
 }
 
+// ---------------------------------------------------------------------------
+// Two transforms of one hidden-size vector in one workgroup: the output transform of a linear
+// layer, the residual addition, the RMSNorm of the next block and the input transform of the
+// next linear layer (all four are separate launches otherwise, each with its own cold operands):
+//   x_new = fp16(residual + fp16(post * scale_out * H (sum of parts)))
+//   xt    = fp16(scale_in * H (pre * fp16(w * fp16(x_new * rsqrt(mean(x_new^2) + eps)))))
+// n = 1024 * EPT is a power of two (both transforms of order 1).  Element e = [wave 4][lane 6][i]
+// (i = log2 EPT register bits).  A transform runs its butterflies over the register bits, the six
+// lane bits, and - after one exchange through LDS that swaps the wave bits with the low four
+// lane bits - the remaining four bits.  The first transform leaves the data in the swapped
+// layout, which is as good as any for the element-wise middle part; the second transform swaps
+// back, so xt is stored in natural order.
+// EPT consecutive elements as floats, with the widest loads the alignment (EPT elements) allows
+template <int EPT>
+__device__ __forceinline__ void ld_f32(const float* p, float v[EPT]) {
+  if constexpr (EPT == 2) {
+    const float2 t = *reinterpret_cast<const float2*>(p);
+    v[0] = t.x;
+    v[1] = t.y;
+  } else {
+#pragma unroll
+    for (int q = 0; q < EPT / 4; ++q) {
+      const float4v t = *reinterpret_cast<const float4v*>(p + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[4 * q + e] = t[e];
+    }
+  }
+}
+template <int EPT>
+__device__ __forceinline__ void ld_f16(const _Float16* p, float v[EPT]) {
+  typedef _Float16 hvec __attribute__((ext_vector_type(EPT)));
+  const hvec t = *reinterpret_cast<const hvec*>(p);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) v[e] = (float)t[e];
+}
+template <int EPT>
+__device__ __forceinline__ void st_f16(_Float16* p, const _Float16 v[EPT]) {
+  typedef _Float16 hvec __attribute__((ext_vector_type(EPT)));
+  hvec t;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) t[e] = v[e];
+  *reinterpret_cast<hvec*>(p) = t;
+}
+
+template <int EPT>
+__device__ __forceinline__ void wht_regs(float v[EPT]) {
+#pragma unroll
+  for (int h = 1; h < EPT; h <<= 1)
+#pragma unroll
+    for (int i = 0; i < EPT; ++i)
+      if (!(i & h)) {
+        const float a = v[i], b = v[i + h];
+        v[i] = a + b;
+        v[i + h] = a - b;
+      }
+}
+
+// exchange buffer index of element e: one pad block of EPT floats per 64 lanes keeps the strided reads apart
+template <int EPT>
+__device__ __forceinline__ int xidx(int e) {
+  return e + EPT * (e / (64 * EPT));
+}
+
+template <int EPT>
+__global__ __launch_bounds__(kRhtThreads) void rht_chain_kernel(
+    _Float16* __restrict__ xt_out, _Float16* __restrict__ x_out, const float* __restrict__ parts,
+    int in_parts, size_t part_stride, const float* __restrict__ post, float scale_out,
+    const _Float16* __restrict__ residual, const _Float16* __restrict__ norm_w, float eps,
+    const _Float16* __restrict__ pre, float scale_in) {
+  constexpr int N = kRhtThreads * EPT;
+  __shared__ __align__(16) float xbuf[N + N / 64];
+  __shared__ float wsum[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const size_t row = blockIdx.x;
+  parts += row * N;
+  // natural layout: e = tid * EPT + i;  swapped layout: wave bits <-> low four lane bits
+  const int e_nat = tid * EPT;
+  const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
+  // ---- operands of the middle part, in the swapped layout (issued first: they are cold)
+  float pv[EPT], rv[EPT], wv[EPT], sv[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) pv[i] = sv[i] = 1.f;
+  if (post) ld_f32<EPT>(post + e_swp, pv);
+  ld_f16<EPT>(residual + row * N + e_swp, rv);
+  ld_f16<EPT>(norm_w + e_swp, wv);
+  if (pre) ld_f16<EPT>(pre + e_swp, sv);
+  // ---- first transform
+  float v[EPT];
+  ld_f32<EPT>(parts + e_nat, v);
+  for (int w = 1; w < in_parts; ++w) {
+    float t[EPT];
+    ld_f32<EPT>(parts + w * part_stride + e_nat, t);
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) v[i] += t[i];
+  }
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_nat + i)] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(xbuf[xidx<EPT>(e_swp + i)], 4, lane);
+  // ---- residual, RMSNorm, sign vector of the next layer
+  float ss = 0.f;
+  _Float16 xn[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    const float o = v[i] * scale_out * pv[i];
+    xn[i] = (_Float16)(rv[i] + (float)(_Float16)o);
+    v[i] = (float)xn[i];
+    ss += v[i] * v[i];
+  }
+  st_f16<EPT>(x_out + row * N + e_swp, xn);
+  ss = wave_sum(ss);
+  if (lane == 0) wsum[wave] = ss;
+  __syncthreads();  // also: every read of xbuf above is done
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) tot += wsum[w];
+  const float rs = __builtin_amdgcn_rsqf(tot / (float)N + eps);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = (float)(_Float16)(wv[i] * (float)(_Float16)(v[i] * rs)) * sv[i];
+  // ---- second transform, from the swapped layout back to the natural one
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_swp + i)] = v[i];
+  __syncthreads();
+  // the bits still missing are the top four of the element's lane field = lane bits 2..5 here
+  _Float16 xo[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    float y = xbuf[xidx<EPT>(e_nat + i)];
+#pragma unroll
+    for (int b = 2; b < 6; ++b) {
+      const float o = lane_xor(y, b);
+      y = ((lane >> b) & 1) ? o - y : y + o;
+    }
+    xo[i] = (_Float16)(y * scale_in);
+  }
+  st_f16<EPT>(xt_out + row * N + e_nat, xo);
+}
+
 }  // namespace
 
 extern "C" {
@@ -628,6 +773,28 @@ int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int i
   P.order = order;
   P.pre_mode = pre_mode;
   return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+int qtip_rht_chain(void* xt_out_f16, void* x_out_f16, const float* parts, int in_parts, int rows, int n,
+                   const float* post_f32, float scale_out, const void* residual_f16,
+                   const void* norm_weight_f16, float eps, const void* pre_f16, float scale_in,
+                   void* stream) {
+  if (!xt_out_f16 || !x_out_f16 || !parts || !residual_f16 || !norm_weight_f16) return QTIP_E_NULL;
+  if (rows < 1 || rows > 65535 || in_parts < 1 || in_parts > kMaxParts) return QTIP_E_SHAPE;
+  if (n != 2048 && n != 4096 && n != 8192) return QTIP_E_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t stride = (size_t)rows * n;
+#define QTIP_CHAIN(E)                                                                              \
+  rht_chain_kernel<E><<<rows, kRhtThreads, 0, st>>>(                                               \
+      (_Float16*)xt_out_f16, (_Float16*)x_out_f16, parts, in_parts, stride, post_f32, scale_out, \
+      (const _Float16*)residual_f16, (const _Float16*)norm_weight_f16, eps, (const _Float16*)pre_f16, scale_in)
+  switch (n) {
+    case 2048: QTIP_CHAIN(2); break;
+    case 4096: QTIP_CHAIN(4); break;
+    default: QTIP_CHAIN(8); break;
+  }
+#undef QTIP_CHAIN
+  return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -131,29 +131,47 @@ class DecoderLayer(nn.Module):
         x = x + self.down(F.silu(gate) * up)
         return x
 
-    def decode_fused(self, x, k_cache, v_cache, pos, inv_freq):
-        """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
-        layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections."""
-        cfg = self.cfg
+    def _fused_linears(self):
         if not hasattr(self, "_fused"):
             names = ('qkv', 'o', 'up_gate', 'down') if self.fused else \
                 ('q_proj', 'k_proj', 'v_proj', 'o', 'gate_proj', 'up_proj', 'down')
             self._fused = {n: _FusedLinear(getattr(self, n)) for n in names}
-        f = self._fused
+        return self._fused
+
+    def decode_fused(self, x, k_cache, v_cache, pos, inv_freq, xt_qkv=None, next_layer=None):
+        """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
+        layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections.
+        With power-of-two hidden sizes the [transform-out + residual] of o / down and the
+        [RMSNorm + transform-in] that follows are one launch (11 per layer): `xt_qkv` is then the
+        already transformed input of this layer's qkv matvec (made by the previous layer) and
+        `next_layer` the layer whose qkv input this one prepares.  Returns (x, xt for the next layer)."""
+        cfg = self.cfg
+        f = self._fused_linears()
         if self.fused:
-            qkv = f['qkv'](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+            if xt_qkv is None:
+                xt_qkv = f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
+            qkv = f['qkv'].transform_out(f['qkv'].matvec(xt_qkv))
         else:
             qkv = torch.cat([f[n](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
                              for n in ('q_proj', 'k_proj', 'v_proj')], dim=-1)
         attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
                                     cfg.head_dim)
-        x = f['o'](attn.reshape(1, -1), residual=x)
-        if self.fused:
-            ug = f['up_gate'](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+        if self.fused and f['o'].can_chain_into(f['up_gate']):
+            parts = f['o'].matvec(f['o'].transform_in(attn.reshape(1, -1)))
+            x, xt_ug = f['o'].chain(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
+            ug = f['up_gate'].transform_out(f['up_gate'].matvec(xt_ug))
         else:
-            ug = torch.cat([f[n](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
-                            for n in ('gate_proj', 'up_proj')], dim=-1)
-        return f['down'](ug, ops.PRE_SILU_MUL, residual=x)
+            x = f['o'](attn.reshape(1, -1), residual=x)
+            if self.fused:
+                ug = f['up_gate'](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+            else:
+                ug = torch.cat([f[n](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
+                                for n in ('gate_proj', 'up_proj')], dim=-1)
+        nq = next_layer._fused_linears().get('qkv') if (next_layer is not None and next_layer.fused) else None
+        if nq is not None and not f['down'].dense and f['down'].can_chain_into(nq):
+            parts = f['down'].matvec(f['down'].transform_in(ug, ops.PRE_SILU_MUL))
+            return f['down'].chain(parts, x, nq, next_layer.input_norm.weight, cfg.eps)
+        return f['down'](ug, ops.PRE_SILU_MUL, residual=x), None
 
 
 class _FusedLinear:
@@ -188,15 +206,34 @@ class _FusedLinear:
         y = self.lin(x)
         return y if residual is None else residual + y
 
-    def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
-        if self.dense:
-            return self._dense(x, pre_mode, norm_weight, eps, residual)
-        xt = ops.rht(x, order=self.Kl, had_bits=self.bl, pre=self.SU, scale=(self.n**-0.5) / 32.0,
-                     out_dtype=torch.float16, pre_mode=pre_mode, norm_weight=norm_weight, eps=eps)
-        parts = ops.decompress_matvec_parts(self.trellis, xt.reshape(-1), self.tlut, self.m, self.n, self.K)
+    def transform_in(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0):
+        return ops.rht(x, order=self.Kl, had_bits=self.bl, pre=self.SU, scale=(self.n**-0.5) / 32.0,
+                       out_dtype=torch.float16, pre_mode=pre_mode, norm_weight=norm_weight, eps=eps)
+
+    def matvec(self, xt):
+        """(S, 1, m) fp32 partial sums."""
+        return ops.decompress_matvec_parts(self.trellis, xt.reshape(-1), self.tlut, self.m, self.n, self.K).unsqueeze(1)
+
+    def transform_out(self, parts, residual=None):
         return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
                        post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
                        residual=residual)
+
+    def can_chain_into(self, nxt):
+        """This layer's output transform and `nxt`'s input transform are plain power-of-two
+        transforms of one hidden-size vector: one launch does both plus residual and RMSNorm."""
+        return (not self.dense and not nxt.dense and self.Kr == 1 and nxt.Kl == 1 and self.m == nxt.n
+                and self.m in (2048, 4096, 8192))
+
+    def chain(self, parts, residual, nxt, norm_weight, eps):
+        """(x_new, xt): transform_out(parts) + residual, then nxt.transform_in(RMSNorm(x_new))."""
+        return ops.rht_chain(parts, self.SV, (self.m**-0.5) * 32.0, residual, norm_weight, eps, nxt.SU,
+                             (nxt.n**-0.5) / 32.0)
+
+    def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
+        if self.dense:
+            return self._dense(x, pre_mode, norm_weight, eps, residual)
+        return self.transform_out(self.matvec(self.transform_in(x, pre_mode, norm_weight, eps)), residual)
 
 
 def _rotate_half(x):
@@ -253,8 +290,10 @@ class LlamaDecoder(nn.Module):
     def decode_fused(self, tok, pos):
         """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab) fp32, fused kernels."""
         x = self.embed[tok.reshape(-1)]
+        xt = None
         for i, layer in enumerate(self.layers):
-            x = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq)
+            nxt = self.layers[i + 1] if i + 1 < len(self.layers) else None
+            x, xt = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq, xt, nxt)
         x = self.norm(x)
         return (x @ self.lm_head.T).float().reshape(1, 1, -1)
 

@@ -316,3 +316,28 @@ def decode_natural(packed, lut, m, n, td_x, td_y, K, V):
         check(lib().qtip_decode_natural(_ptr(out), _ptr(packed), _ptr(lut), _DT[lut.dtype], m, n, td_x, td_y, K, V,
                                         stream_ptr(packed.device)), "qtip_decode_natural")
     return out
+
+
+def rht_chain(parts, post, scale_out, residual, norm_weight, eps, pre, scale_in):
+    """(x_new, xt) for one hidden-size vector per row, one launch:
+    x_new = fp16(residual + fp16(post * scale_out * H(sum(parts)))),
+    xt = fp16(scale_in * H(pre * rmsnorm(x_new))).  parts: (S, rows, n) fp32, n in {2048, 4096, 8192}."""
+    require_cuda(parts, "parts", torch.float32)
+    require_cuda(residual, "residual", torch.float16)
+    require_cuda(norm_weight, "norm_weight", torch.float16)
+    if parts.dim() != 3:
+        raise ValueError("parts must be (S, rows, n)")
+    S, rows, n = parts.shape
+    if n not in (2048, 4096, 8192) or residual.numel() != rows * n or norm_weight.numel() != n:
+        raise ValueError("rht_chain: unsupported or inconsistent shapes")
+    if post is not None:
+        require_cuda(post, "post", torch.float32)
+    if pre is not None:
+        require_cuda(pre, "pre", torch.float16)
+    x_new = torch.empty((rows, n), dtype=torch.float16, device=parts.device)
+    xt = torch.empty((rows, n), dtype=torch.float16, device=parts.device)
+    with torch.cuda.device(parts.device):
+        check(lib().qtip_rht_chain(_ptr(xt), _ptr(x_new), _ptr(parts), S, rows, n, _ptr(post), ctypes.c_float(scale_out),
+                                   _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(pre),
+                                   ctypes.c_float(scale_in), stream_ptr(parts.device)), "qtip_rht_chain")
+    return x_new, xt

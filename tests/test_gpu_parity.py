@@ -412,3 +412,34 @@ def test_fused_decode_step_matches_generic():
     assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
     for c0, c1 in zip(kc, model.k_cache):
         assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 8192])
+@pytest.mark.parametrize("S,rows", [(1, 1), (2, 1), (4, 3)])
+def test_rht_chain_matches_two_launches(n, S, rows):
+    """[transform-out + residual] + [RMSNorm + transform-in] in one workgroup against the two fused
+    launches it replaces, and against a float64 statement of the same rounding sequence."""
+    from qtip_amd import ops
+    g = torch.Generator().manual_seed(n + S + rows)
+    parts = torch.randn(S, rows, n, generator=g).cuda()
+    SV = (torch.sign(torch.randn(n, generator=g)) * (0.5 + torch.rand(n, generator=g))).cuda()
+    SU = torch.sign(torch.randn(n, generator=g)).half().cuda()
+    res = torch.randn(rows, n, generator=g).half().cuda()
+    w = (1 + 0.1 * torch.randn(n, generator=g)).half().cuda()
+    so, si, eps = 32.0 * n**-0.5, n**-0.5 / 32.0, 1e-5
+    x_new, xt = ops.rht_chain(parts, SV, so, res, w, eps, SU, si)
+    x_ref = ops.rht(parts, post=SV, scale=so, out_dtype=torch.float16, in_parts=S, residual=res)
+    xt_ref = ops.rht(x_ref, pre=SU, scale=si, out_dtype=torch.float16, pre_mode=ops.PRE_RMSNORM, norm_weight=w, eps=eps)
+    # fp32 sums in another order: results agree to an fp16 ulp here and there
+    assert (x_new.float() - x_ref.float()).abs().max() <= 2e-3 * x_ref.float().abs().max()
+    assert (xt.float() - xt_ref.float()).abs().max() <= 4e-3 * xt_ref.float().abs().max()
+    # independent float64 statement
+    H = O.hadamard_transform(np.eye(n))  # symmetric for powers of two
+    y = (parts.double().sum(0).cpu().numpy() @ H) * SV.double().cpu().numpy() * (so * n**0.5)
+    xn = (res.float().cpu().numpy() + y.astype(np.float16).astype(np.float32)).astype(np.float16)
+    assert np.abs(x_new.float().cpu().numpy() - xn.astype(np.float32)).max() <= 2e-3 * np.abs(xn).max()
+    v = xn.astype(np.float64)
+    rs = 1.0 / np.sqrt((v**2).mean(-1, keepdims=True) + eps)
+    hn = (w.float().cpu().numpy() * (v * rs).astype(np.float16).astype(np.float32)).astype(np.float16).astype(np.float64)
+    t = ((hn * SU.float().cpu().numpy()) @ H) * (si * n**0.5)
+    assert np.abs(xt.float().cpu().numpy() - t).max() <= 4e-3 * np.abs(t).max()
