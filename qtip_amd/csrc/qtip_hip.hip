@@ -174,7 +174,8 @@ __device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t
 // count in every unit).  DEPTH items are in flight; the prefetch runs ahead
 // across unit boundaries and every load in the loop is unconditional (a
 // conditional prefetch makes the compiler wait for it at once): padding items
-// fetch offset 0 and are skipped by the arithmetic.
+// use an out-of-range lane offset (the load returns zeros without a memory
+// access) and are skipped by the arithmetic.
 // XLDS: the x values of the workgroup's k range are staged in LDS once
 // (needs 256 bytes per wave-load of the range) and read from there.
 template <int K, int DEPTH, bool XLDS>
@@ -228,8 +229,11 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     const uint32_t wl = (uint32_t)(w_first + l_j * kWaves);
     const uint32_t woff = valid ? l_rboff + wl * WL_BYTES : 0u;
     const uint32_t xw = valid ? wl * 256u : 0u;
-    buf[d] = load_lane_buf<K>(rs_w, loff, woff);
-    if constexpr (!XLDS) load_x_buf(rs_x, xoff, xw, xbuf[d]);
+    // padding items: a lane offset past the end of the descriptor returns zeros without touching
+    // memory (reading offset 0 instead cost the small shapes up to 2 us: thousands of waves
+    // hammering the same few cache lines)
+    buf[d] = load_lane_buf<K>(rs_w, valid ? loff : 0x7FFFFF00u, woff);
+    if constexpr (!XLDS) load_x_buf(rs_x, valid ? xoff : 0x7FFFFF00u, xw, xbuf[d]);
     ++l_t;
     if (++l_j == npw) {
       l_j = 0;
@@ -273,6 +277,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     }
   }
   __syncthreads();
+
   const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)wave * 256u;  // wave-load w_first
 
   float4_t acc[4];  // [2*mh + rh]: rows 16*mh + 8*rh + a/2 of the unit's 32-row block
@@ -430,7 +435,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
     const int rb = l_grp * kGemmRB + rbi;
     const int wl = wl0 + KS * l_t + ks;
     const bool valid = l_q < T && rb < nrb && wl < wl1;
-    buf[d] = load_lane_buf<K>(rs_w, loff, valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u);
+    buf[d] = load_lane_buf<K>(rs_w, valid ? loff : 0x7FFFFF00u,  // padding: out of range, no memory access
+                              valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u);
     ++l_q;
     if (++l_t == nst) {
       l_t = 0;
@@ -712,7 +718,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
     const long rounds = (units + cus - 1) / cus;
     const double per_unit = (double)nwl / S + 12.0 + (S > 1 ? 4.0 : 0.0);
     double cost = rounds * per_unit;
-    if (cost < 60.0) cost = 60.0;
+    if (cost < 40.0) cost = 40.0;
     if (S > 1 && summed) cost += 53.0;
     if (cost < best_cost * 0.97) {
       best_cost = cost;
