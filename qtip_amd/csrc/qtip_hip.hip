@@ -447,6 +447,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
   for (int d = 0; d < DEPTH; ++d) issue(d);
 
   // ---- activation tiles: thread fills NB 16-byte chunks per tile
+  static_assert(DEPTH % 2 == 0, "stage parity must be static inside the unrolled loop");
   u32x4 xg[2][NB];  // tiles on their way: [parity of the stage][chunk]
   auto load_tile = [&](int slot, int t) {  // stage t of a unit -> registers
     const int col0 = 128 * (wl0 + KS * t);
@@ -680,8 +681,8 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 1, 3, 16>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 2, 3, 8>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
+    QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
 #undef QTIP_ALLOW
@@ -915,7 +916,7 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
     const int rnd = Sp > 1 ? 0 : round_f16;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
 #define QTIP_GEMM(KB, NBT, WV)                                                                          \
-  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? 3 : 2), WV><<<(int)grid, WV * 64, kGemmLds, st>>>(      \
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? (WV == 16 ? 2 : 4) : 2), WV><<<(int)grid, WV * 64, kGemmLds, st>>>( \
       d, p, xx, t, m, k, nb, rnd, Sp, wl_per)
 #define QTIP_GEMM_K(KB)               \
   if (nb <= 16) QTIP_GEMM(KB, 1, 16); \
