@@ -14,14 +14,16 @@ from ._lib import QTIP_F16, QTIP_F32, check, lib, require_cuda, stream_ptr
 
 _DT = {torch.float16: QTIP_F16, torch.float32: QTIP_F32}
 
-# per-device scratch for the partial sums of the split-k matvec
+# scratch for split-k partial sums, one buffer per (device, stream): launches on one stream are
+# ordered, launches on different streams must not share partial results
 _WORKSPACE = {}
 _WORKSPACE_BYTES = 8 << 20
 _SPLIT = {}
 
 
 def _workspace(device, need):
-    key = device.index if device.index is not None else torch.cuda.current_device()
+    dev = device.index if device.index is not None else torch.cuda.current_device()
+    key = (dev, torch.cuda.current_stream(device).cuda_stream)
     ws = _WORKSPACE.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.empty(max(need, _WORKSPACE_BYTES), dtype=torch.uint8, device=device)
