@@ -68,10 +68,6 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // decompress + matvec
 // ---------------------------------------------------------------------------
 constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
-#ifndef QTIP_D2X
-#define QTIP_D2X 6
-#endif
-constexpr int kD2X = QTIP_D2X;
 constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a workgroup's k range
 
 // index into W[32] (lookup order of matvec_accumulate) of state (R, t, j)
@@ -126,10 +122,7 @@ template <int K>
 __device__ __forceinline__ LaneData<K> load_lane_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
                                                      uint32_t soff) {
   LaneData<K> r;
-#ifndef QTIP_NT
-#define QTIP_NT 2
-#endif
-  constexpr int NT = QTIP_NT;  // non-temporal: the stream is read once
+  constexpr int NT = 2;  // non-temporal: the stream is read once
   if constexpr (K == 2) {
     const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
 #pragma unroll
@@ -676,7 +669,7 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 4, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<3, 3, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<2, kD2X, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
@@ -802,7 +795,7 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {
-      case 2: matvec_kernel<2, kD2X, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, 6, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
       case 3: matvec_kernel<3, 4, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
       default: matvec_kernel<4, 3, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
     }

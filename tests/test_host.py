@@ -71,7 +71,7 @@ def test_has_kernel_gate():
 
 def test_op_registry_names():
     import qtip_amd.codebook as cbk
-    # every BASELINE shape at every bit width, under the reference's naming scheme
+    # every Llama-2 7B / 70B layer shape at every bit width, under the reference's naming scheme
     for m, k in [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (10240, 8192), (8192, 8192),
                  (57344, 8192), (8192, 28672), (28672, 8192)]:
         for b in (2, 3, 4):
