@@ -48,7 +48,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
     ap.add_argument("--extras", default="shapes,layer,gemm,e2e",
-                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, e2e "
+                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, e2e, e2e70b "
                          "(counter runs under rocprofv3 pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
@@ -229,6 +229,20 @@ def main():
         result["e2e_decode"] = {"model": "Llama-2-7B architecture, random init, 2-bit HYB, fused qkv and up/gate",
                                 "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1),
                                 "ms_per_token": round(1e3 / tps, 3)}
+        del model
+        torch.cuda.empty_cache()
+
+    if "e2e70b" in extras:
+        # the same loop on the Llama-2-70B architecture (80 layers, GQA 64/8 heads, 17 GB of 2-bit weights);
+        # not part of the default run: building the random model takes a minute
+        from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+        cfg70 = LlamaConfig(hidden=8192, heads=64, kv_heads=8, layers=80, ffn=28672, vocab=32000, K=2)
+        model = LlamaDecoder(cfg70, max_cache_len=512, device=dev)
+        prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
+        _, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
+        result["e2e_decode_70b"] = {"model": "Llama-2-70B architecture, random init, 2-bit HYB, fused qkv and up/gate",
+                                    "prompt": 128, "new_tokens": 128, "tok_per_s": round(tps, 1),
+                                    "ms_per_token": round(1e3 / tps, 3)}
         del model
         torch.cuda.empty_cache()
 
