@@ -443,3 +443,36 @@ def test_rht_chain_matches_two_launches(n, S, rows):
     hn = (w.float().cpu().numpy() * (v * rs).astype(np.float16).astype(np.float32)).astype(np.float16).astype(np.float64)
     t = ((hn * SU.float().cpu().numpy()) @ H) * (si * n**0.5)
     assert np.abs(xt.float().cpu().numpy() - t).max() <= 4e-3 * np.abs(t).max()
+
+
+@pytest.mark.parametrize("rcp", [1, 2])
+@pytest.mark.parametrize("bs", [1, 3])
+def test_forward_with_per_shard_transforms(rcp, bs):
+    """rcp 1 / 2: the input / output transform acts on each of the tp_rank shards of the vector
+    separately (lib/codebook/bitshift.py:437-441, 465-469), as layers quantised for tensor
+    parallelism expect."""
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    m, k, K, shards = 512, 1536, 2, 8   # 1536 = 12 * 128, shard 192 = 12 * 16; 512 / 8 = 64
+    L = make_layer(m, k, K, seed=rcp)
+    mod = BitshiftLinear(16, 16, 16, K, 2, 9, "quantlut_sym", tlut=dev(L["tlut"]), has_kernel=True)
+    g = torch.Generator().manual_seed(bs)
+    x = torch.randn(bs, k, generator=g).half()
+    hl, Kl = mh.get_hadK(k)
+    hr, Kr = mh.get_hadK(m)
+    y = mod(x.cuda(), dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), hl, hr, Kl, Kr, rcp, shards).float().cpu().numpy()
+    W = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float64)
+    xs = x.numpy().astype(np.float64) * L["SU"].astype(np.float64)
+    if rcp == 1:
+        xt = O.hadamard_transform(xs.reshape(-1, k // shards), transpose=True).reshape(bs, k) / 32
+    else:
+        xt = O.hadamard_transform(xs, transpose=True) / 32
+    z = xt.astype(np.float16).astype(np.float64) @ W.T
+    if bs > 1:
+        z = z.astype(np.float16).astype(np.float64)  # the batched path returns an fp16 product
+    if rcp == 2:
+        z = O.hadamard_transform(z.reshape(-1, m // shards)).reshape(bs, m)
+    else:
+        z = O.hadamard_transform(z)
+    ref = z * (L["SV"].astype(np.float64) * 32)
+    assert_close(y, ref, max_rel=1e-2, mean_rel=2e-3)
