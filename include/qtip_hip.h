@@ -87,6 +87,17 @@ int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x
                                  const void* tlut, int m, int k, int bits, int nparts,
                                  void* stream);
 
+/* qtip_decompress_matvec_parts with the input transform of the layer inside the kernel:
+ *   x_t = fp16(scale * H_k (su * x_raw)),  parts = hatW . x_t
+ * i.e. matmul_hadUt_cuda + the SU multiply + the fp16 cast of BitshiftLinear.forward
+ * (lib/codebook/bitshift.py:428-441, lib/utils/matmul_had.py:92-119) and the matvec in one
+ * launch.  k in {2048, 4096, 8192} (power-of-two transform, order 1); x_raw and su are
+ * fp16[k], 16-byte aligned; scale is 1/sqrt(k)/32 in the forward pass.  Every workgroup
+ * computes the whole transform while its first weight loads are in flight. */
+int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const void* x_raw_f16,
+                                     const void* su_f16, float scale, const void* tlut, int m, int k,
+                                     int bits, int nparts, void* stream);
+
 /* Bytes of scratch qtip_decompress_gemm wants for this shape (0 when it does not split k). */
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch);
 

@@ -256,7 +256,12 @@ class BitshiftLinear(nn.Module):
 
         # ---- input transform: fp16(H_L^T (x * SU) / sqrt(n) / 32)
         fused_in = (rcp != 1 and SU.dtype == torch.float16 and x.dtype in (torch.float16, torch.float32))
-        if fused_in:
+        # one token, power-of-two input size: the matvec kernel transforms its input itself
+        in_matvec = (fused_in and bs == 1 and self.has_kernel and K_left == 1 and x.dtype == torch.float16
+                     and n in ops.RHT_IN_MATVEC_SIZES)
+        if in_matvec:
+            xt = None
+        elif fused_in:
             xt = ops.rht(x.contiguous(), order=K_left,
                          had_bits=had_bits(had_left, K_left, True, dev) if K_left > 1 else None,
                          pre=SU.contiguous(), scale=(n**-0.5) / self.scale, out_dtype=torch.float16)
@@ -273,7 +278,11 @@ class BitshiftLinear(nn.Module):
         in_parts = 1
         if self.has_kernel:
             tl = self._tlut16(dev)
-            if bs == 1:
+            if in_matvec:
+                y = ops.decompress_matvec_parts_rht(trellis.reshape(-1), x.reshape(-1), SU.contiguous(),
+                                                    (n**-0.5) / self.scale, tl.reshape(-1), m, n, self.cb.K)
+                in_parts = y.shape[0]
+            elif bs == 1:
                 # same kernel as the quip_lib::decompress_matvec_qtip_* op; the k-split
                 # partial sums (if any) are added by the output transform on load
                 y = ops.decompress_matvec_parts(trellis.reshape(-1), xt.reshape(-1), tl.reshape(-1), m, n, self.cb.K)

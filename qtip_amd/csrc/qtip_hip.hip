@@ -6,6 +6,7 @@
 
 #include "../../include/qtip_hip.h"
 #include "qtip_device.h"
+#include "qtip_wht.h"
 
 using namespace qtip;
 
@@ -153,6 +154,35 @@ __device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t
   for (int q = 0; q < 4; ++q) xv[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff + 16 * q, soff, 0);
 }
 
+// Input transform of the layer inside the matvec prologue (k = 1024 * EPT a power of two):
+// xs[e] = fp16(scale * (H_k (su * x))[e]) for the whole vector, written to LDS where the
+// kernel keeps its activations.  Every workgroup computes the whole transform (a few thousand
+// butterflies per thread, hidden behind the latency of the first weight loads) - it replaces
+// a separate transform launch.  `scratch` (k + k/64 floats) is the table's LDS, not yet built.
+// Element e = [wave 4][lane 6][i]: butterflies over the register bits, the six lane bits and,
+// after one exchange through LDS that swaps the wave bits with the low four lane bits, the rest.
+template <int EPT>
+__device__ __forceinline__ void xform_prologue(const float v_in[8], float scale, float* scratch,
+                                               _Float16* xs, int tid, int lane, int wave) {
+  using namespace qtip_wht;
+  float v[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = v_in[i];
+  const int e_nat = tid * EPT;
+  const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) scratch[xidx<EPT>(e_nat + i)] = v[i];
+  __syncthreads();
+  _Float16 o[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) o[i] = (_Float16)(wht_lanes(scratch[xidx<EPT>(e_swp + i)], 4, lane) * scale);
+  st_f16<EPT>(xs + e_swp, o);
+  __syncthreads();  // scratch is free for the table, xs is complete
+}
+
 // Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup take
 // the unit's wave-loads round-robin (so the workgroup streams one contiguous
 // run of bytes), reduce across the four blocks of a wave-load inside the MFMA, across the two
@@ -171,10 +201,12 @@ __device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t
 // access) and are skipped by the arithmetic.
 // XLDS: the x values of the workgroup's k range are staged in LDS once
 // (needs 256 bytes per wave-load of the range) and read from there.
-template <int K, int DEPTH, bool XLDS>
+template <int K, int DEPTH, bool XLDS, bool XFORM = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int S, int wl_per) {
+    const uint32_t* __restrict__ tlut, int m, int k, int S, int wl_per,
+    const uint16_t* __restrict__ su = nullptr, float xscale = 1.f) {
+  static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
   float* part = reinterpret_cast<float*>(smem + kLut128Bytes);  // [2][kWaves][32]
@@ -241,7 +273,21 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
   for (int it = 0; it < 4; ++it) tw[it] = tlut[it * 128 + (tid >> 3)];
   u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-  if constexpr (XLDS) {
+  float xraw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if constexpr (XFORM) {
+    // the raw activations and the sign vector of the layer, k / 1024 consecutive elements per thread
+    using namespace qtip_wht;
+    float sv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const _Float16* xr = reinterpret_cast<const _Float16*>(x);
+    const _Float16* sr = reinterpret_cast<const _Float16*>(su);
+    switch (k >> 10) {
+      case 2: ld_f16<2>(xr + tid * 2, xraw); ld_f16<2>(sr + tid * 2, sv); break;
+      case 4: ld_f16<4>(xr + tid * 4, xraw); ld_f16<4>(sr + tid * 4, sv); break;
+      default: ld_f16<8>(xr + tid * 8, xraw); ld_f16<8>(sr + tid * 8, sv); break;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xraw[i] *= sv[i];  // entries past k / 1024 are never read
+  } else if constexpr (XLDS) {
     // x of wave-loads [wl0, wl1): 16 bytes per thread and pass, at most 2 passes (28 KiB)
     const int xbytes = (wl1 - wl0) * 256;
     const int kbytes = k * 2;
@@ -255,13 +301,22 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) issue(d);
 
+  if constexpr (XFORM) {
+    float* scratch = reinterpret_cast<float*>(smem);
+    _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
+    switch (k >> 10) {
+      case 2: xform_prologue<2>(xraw, xscale, scratch, xs, tid, lane, wave); break;
+      case 4: xform_prologue<4>(xraw, xscale, scratch, xs, tid, lane, wave); break;
+      default: xform_prologue<8>(xraw, xscale, scratch, xs, tid, lane, wave); break;
+    }
+  }
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const uint32_t w = tw[it & 3] ^ ((uint32_t)(it >> 2) << 15);
     const u32x4 v = {w, w, w, w};
     reinterpret_cast<u32x4*>(lut)[it * kThreads + tid] = v;
   }
-  if constexpr (XLDS) {
+  if constexpr (XLDS && !XFORM) {
     const int xbytes = (wl1 - wl0) * 256;
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps) {
@@ -271,7 +326,8 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   }
   __syncthreads();
 
-  const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)wave * 256u;  // wave-load w_first
+  // wave-load w_first (the transformed vector is stored whole, a staged one from wl0 on)
+  const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)(XFORM ? w_first : wave) * 256u;
 
   float4_t acc[4];  // [2*mh + rh]: rows 16*mh + 8*rh + a/2 of the unit's 32-row block
 #pragma unroll
@@ -672,6 +728,9 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 6, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 4, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 3, true, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
@@ -726,7 +785,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 6; }
+int qtip_abi_version(void) { return 7; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -781,7 +840,8 @@ size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
 }
 
 static int launch_matvec(float* dst, const void* packed, const void* x_f16, const void* tlut, int m,
-                         int k, int bits, int S, hipStream_t st) {
+                         int k, int bits, int S, hipStream_t st, const void* su_f16 = nullptr,
+                         float xscale = 1.f) {
   DeviceInfo& di = device_info();
   const long units = (long)(m >> 5) * S;
   long grid = units < di.cus ? units : di.cus;
@@ -791,6 +851,17 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   auto* p = (const uint8_t*)packed;
   auto* xx = (const uint16_t*)x_f16;
   auto* t = (const uint32_t*)tlut;
+  if (su_f16) {
+    // input transform inside the prologue: the whole transformed vector lives in LDS
+    const size_t lds = kMatvecLds + (size_t)k * 2;
+    auto* sg = (const uint16_t*)su_f16;
+    switch (bits) {
+      case 2: matvec_kernel<2, 6, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      case 3: matvec_kernel<3, 4, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      default: matvec_kernel<4, 3, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+    }
+    return (int)hipGetLastError();
+  }
   const size_t xbytes = (size_t)wl_per * 256;
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
@@ -828,6 +899,18 @@ int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x
   if (rc) return rc;
   if (nparts < 1 || nparts > kMaxSplit || nparts > ((((k >> 5) + 3) >> 2))) return QTIP_E_SHAPE;
   return launch_matvec(parts, packed, x_f16, tlut, m, k, bits, nparts, (hipStream_t)stream);
+}
+
+int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const void* x_raw_f16,
+                                     const void* su_f16, float scale, const void* tlut, int m, int k,
+                                     int bits, int nparts, void* stream) {
+  int rc = check_matvec(parts, packed, x_raw_f16, tlut, m, k, bits);
+  if (rc) return rc;
+  if (!su_f16) return QTIP_E_NULL;
+  if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
+  if (!aligned16(x_raw_f16) || !aligned16(su_f16)) return QTIP_E_ALIGN;
+  return launch_matvec(parts, packed, x_raw_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale);
 }
 
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,

@@ -4,6 +4,9 @@
 #include <stdint.h>
 
 #include "../../include/qtip_hip.h"
+#include "qtip_wht.h"
+
+using namespace qtip_wht;
 
 namespace {
 
@@ -51,45 +54,6 @@ __device__ __forceinline__ float ldf<float>(const float* p, size_t i) {
 template <>
 __device__ __forceinline__ float ldf<_Float16>(const _Float16* p, size_t i) {
   return (float)p[i];
-}
-
-// value of lane ^ (1 << b) for b = 0..5
-__device__ __forceinline__ float lane_xor(float v, int b) {
-  const int u = __builtin_bit_cast(int, v);
-  int r;
-  switch (b) {
-    case 0: r = __builtin_amdgcn_update_dpp(0, u, 0xB1, 0xF, 0xF, false); break;  // quad_perm 1,0,3,2
-    case 1: r = __builtin_amdgcn_update_dpp(0, u, 0x4E, 0xF, 0xF, false); break;  // quad_perm 2,3,0,1
-    case 2:  // xor 4 inside a row of 16: row_ror:12 brings lane+4 to the banks with bit 2 clear, row_ror:4 lane-4 to the others
-      r = __builtin_amdgcn_update_dpp(0, u, 0x12C, 0xF, 0x5, false);
-      r = __builtin_amdgcn_update_dpp(r, u, 0x124, 0xF, 0xA, false);
-      break;
-    case 3: r = __builtin_amdgcn_update_dpp(0, u, 0x128, 0xF, 0xF, false); break;  // xor 8 = row_ror:8
-    case 4: r = __builtin_amdgcn_ds_swizzle(u, 0x401F); break;                    // xor 16
-    default: {
-      auto sw = __builtin_amdgcn_permlane32_swap((uint32_t)u, (uint32_t)u, false, false);
-      r = (int)((threadIdx.x & 32) ? sw[0] : sw[1]);
-    }
-  }
-  return __builtin_bit_cast(float, r);
-}
-
-// Walsh-Hadamard butterflies over lane bits 0 .. nbits-1 (natural order)
-__device__ __forceinline__ float wht_lanes(float v, int nbits, int lane) {
-#pragma unroll
-  for (int b = 0; b < 6; ++b) {
-    if (b < nbits) {
-      const float o = lane_xor(v, b);
-      v = ((lane >> b) & 1) ? o - v : v + o;
-    }
-  }
-  return v;
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int b = 0; b < 6; ++b) v += lane_xor(v, b);
-  return v;
 }
 
 // CH = loads in flight per thread and pass; FUSED enables the prologue modes
@@ -595,57 +559,6 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
 // lane bits - the remaining four bits.  The first transform leaves the data in the swapped
 // layout, which is as good as any for the element-wise middle part; the second transform swaps
 // back, so xt is stored in natural order.
-// EPT consecutive elements as floats, with the widest loads the alignment (EPT elements) allows
-template <int EPT>
-__device__ __forceinline__ void ld_f32(const float* p, float v[EPT]) {
-  if constexpr (EPT == 2) {
-    const float2 t = *reinterpret_cast<const float2*>(p);
-    v[0] = t.x;
-    v[1] = t.y;
-  } else {
-#pragma unroll
-    for (int q = 0; q < EPT / 4; ++q) {
-      const float4v t = *reinterpret_cast<const float4v*>(p + 4 * q);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[4 * q + e] = t[e];
-    }
-  }
-}
-template <int EPT>
-__device__ __forceinline__ void ld_f16(const _Float16* p, float v[EPT]) {
-  typedef _Float16 hvec __attribute__((ext_vector_type(EPT)));
-  const hvec t = *reinterpret_cast<const hvec*>(p);
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) v[e] = (float)t[e];
-}
-template <int EPT>
-__device__ __forceinline__ void st_f16(_Float16* p, const _Float16 v[EPT]) {
-  typedef _Float16 hvec __attribute__((ext_vector_type(EPT)));
-  hvec t;
-#pragma unroll
-  for (int e = 0; e < EPT; ++e) t[e] = v[e];
-  *reinterpret_cast<hvec*>(p) = t;
-}
-
-template <int EPT>
-__device__ __forceinline__ void wht_regs(float v[EPT]) {
-#pragma unroll
-  for (int h = 1; h < EPT; h <<= 1)
-#pragma unroll
-    for (int i = 0; i < EPT; ++i)
-      if (!(i & h)) {
-        const float a = v[i], b = v[i + h];
-        v[i] = a + b;
-        v[i + h] = a - b;
-      }
-}
-
-// exchange buffer index of element e: one pad block of EPT floats per 64 lanes keeps the strided reads apart
-template <int EPT>
-__device__ __forceinline__ int xidx(int e) {
-  return e + EPT * (e / (64 * EPT));
-}
-
 template <int EPT>
 __global__ __launch_bounds__(kRhtThreads) void rht_chain_kernel(
     _Float16* __restrict__ xt_out, _Float16* __restrict__ x_out, const float* __restrict__ parts,

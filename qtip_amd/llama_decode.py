@@ -142,7 +142,8 @@ class DecoderLayer(nn.Module):
         """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
         layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections.
         With power-of-two hidden sizes the [transform-out + residual] of o / down and the
-        [RMSNorm + transform-in] that follows are one launch (11 per layer): `xt_qkv` is then the
+        [RMSNorm + transform-in] that follows are one launch and the o projection transforms its
+        input inside the matvec (10 per layer): `xt_qkv` is then the
         already transformed input of this layer's qkv matvec (made by the previous layer) and
         `next_layer` the layer whose qkv input this one prepares.  Returns (x, xt for the next layer)."""
         cfg = self.cfg
@@ -157,7 +158,7 @@ class DecoderLayer(nn.Module):
         attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
                                     cfg.head_dim)
         if self.fused and f['o'].can_chain_into(f['up_gate']):
-            parts = f['o'].matvec(f['o'].transform_in(attn.reshape(1, -1)))
+            parts = f['o'].matvec_from(attn.reshape(1, -1))
             x, xt_ug = f['o'].chain(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
             ug = f['up_gate'].transform_out(f['up_gate'].matvec(xt_ug))
         else:
@@ -214,6 +215,15 @@ class _FusedLinear:
         """(S, 1, m) fp32 partial sums."""
         return ops.decompress_matvec_parts(self.trellis, xt.reshape(-1), self.tlut, self.m, self.n, self.K).unsqueeze(1)
 
+    def matvec_from(self, x):
+        """matvec(transform_in(x)) for a plain input; one launch when the transform is a power of
+        two the matvec kernel computes in its prologue."""
+        if (self.Kl == 1 and self.n in ops.RHT_IN_MATVEC_SIZES and x.dtype == torch.float16
+                and self.SU.dtype == torch.float16):
+            return ops.decompress_matvec_parts_rht(self.trellis, x.reshape(-1), self.SU, (self.n**-0.5) / 32.0,
+                                                   self.tlut, self.m, self.n, self.K).unsqueeze(1)
+        return self.matvec(self.transform_in(x))
+
     def transform_out(self, parts, residual=None):
         return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
                        post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
@@ -233,6 +243,8 @@ class _FusedLinear:
     def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
         if self.dense:
             return self._dense(x, pre_mode, norm_weight, eps, residual)
+        if pre_mode == ops.PRE_NONE:
+            return self.transform_out(self.matvec_from(x), residual)
         return self.transform_out(self.matvec(self.transform_in(x, pre_mode, norm_weight, eps)), residual)
 
 

@@ -119,6 +119,29 @@ def decompress_matvec_parts(packed, x, tlut, m, k, bits, nparts=None):
     return parts
 
 
+RHT_IN_MATVEC_SIZES = (2048, 4096, 8192)
+
+
+def decompress_matvec_parts_rht(packed, x_raw, su, scale, tlut, m, k, bits, nparts=None):
+    """(S, m) fp32 partial sums of decode(packed) @ fp16(scale * H_k(su * x_raw)): the input
+    transform of the layer runs inside the matvec launch (k in RHT_IN_MATVEC_SIZES)."""
+    _check_packed(packed, m, k, bits)
+    _check_tlut(tlut, packed.device)
+    require_cuda(x_raw, "x", torch.float16)
+    require_cuda(su, "su", torch.float16)
+    if k not in RHT_IN_MATVEC_SIZES or x_raw.numel() != k or su.numel() != k:
+        raise ValueError(f"x and su must hold k = {k} fp16 values, k in {RHT_IN_MATVEC_SIZES}")
+    if x_raw.device != packed.device or su.device != packed.device:
+        raise ValueError(f"x and su must be on {packed.device}")
+    S = int(nparts) if nparts is not None else matvec_split(m, k, bits, packed.device)
+    parts = torch.empty((S, m), dtype=torch.float32, device=packed.device)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_decompress_matvec_parts_rht(_ptr(parts), _ptr(packed), _ptr(x_raw), _ptr(su),
+                                                     ctypes.c_float(scale), _ptr(tlut), m, k, bits, S,
+                                                     stream_ptr(packed.device)), "qtip_decompress_matvec_parts_rht")
+    return parts
+
+
 def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     """(batch, m) fp32 = x[batch,k] (fp16) @ decode(packed)[m,k]^T on the matrix cores."""
     _check_packed(packed, m, k, bits)

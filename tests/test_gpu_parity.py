@@ -445,6 +445,34 @@ def test_rht_chain_matches_two_launches(n, S, rows):
     assert np.abs(xt.float().cpu().numpy() - t).max() <= 4e-3 * np.abs(t).max()
 
 
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("m,k,S", [(256, 2048, None), (1024, 4096, 1), (4096, 4096, None), (512, 8192, 4),
+                                   (2048, 8192, None)])
+def test_matvec_with_transform_in_prologue(K, m, k, S):
+    """The matvec that computes fp16(scale * H_k(su * x)) itself against the transform launch
+    followed by the plain matvec (same partial-sum layout), and against a float64 statement."""
+    from qtip_amd import ops
+    L = make_layer(m, k, K, seed=m + k + K)
+    g = torch.Generator().manual_seed(K + m)
+    x = torch.randn(k, generator=g).half().cuda()
+    su = dev(L["SU"]).half()
+    scale = k**-0.5 / 32.0
+    packed, tlut = dev(L["packed"]).reshape(-1), dev(L["tlut"]).reshape(-1)
+    parts = ops.decompress_matvec_parts_rht(packed, x, su, scale, tlut, m, k, K, nparts=S)
+    xt = ops.rht(x.reshape(1, k), pre=su, scale=scale, out_dtype=torch.float16)
+    ref = ops.decompress_matvec_parts(packed, xt.reshape(-1), tlut, m, k, K, nparts=S)
+    assert parts.shape == ref.shape
+    y, r = parts.sum(0).double().cpu().numpy(), ref.sum(0).double().cpu().numpy()
+    # the butterflies run in another order: x_t differs by an fp16 ulp in a few places
+    assert np.abs(y - r).max() <= 2e-3 * np.abs(r).max()
+    W = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float64)
+    H = O.hadamard_transform(np.eye(k))
+    t = ((x.double().cpu().numpy() * su.double().cpu().numpy()) @ H) * (scale * k**0.5)
+    t16 = t.astype(np.float16).astype(np.float64)
+    want = W @ t16
+    assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("rcp", [1, 2])
 @pytest.mark.parametrize("bs", [1, 3])
 def test_forward_with_per_shard_transforms(rcp, bs):
