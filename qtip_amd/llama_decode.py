@@ -310,21 +310,54 @@ class LlamaDecoder(nn.Module):
         return (x @ self.lm_head.T).float().reshape(1, 1, -1)
 
 
+def logits_to_probs(logits, temperature=1.0, top_k=None):
+    """softmax(logits / temperature) restricted to the top_k largest logits
+    (eval/interactive_gen.py:23-33)."""
+    logits = logits / max(temperature, 1e-5)
+    if top_k is not None:
+        v, _ = torch.topk(logits, min(top_k, logits.size(-1)))
+        logits = torch.where(logits < v[..., -1:], float("-inf"), logits)
+    return torch.softmax(logits, dim=-1)
+
+
+def sample(logits, temperature=1.0, top_k=None):
+    """One token per row from the last position's distribution, without a host
+    synchronisation: argmax(p / Exp(1)) draws from p (eval/interactive_gen.py:15-40)."""
+    probs = logits_to_probs(logits[:, -1], temperature, top_k)
+    q = torch.empty_like(probs).exponential_(1)
+    return torch.argmax(probs / q, dim=-1, keepdim=True), probs
+
+
 @torch.no_grad()
-def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True):
-    """Greedy decode.  Returns (token ids, decode seconds, tokens per second);
-    throughput is max_new_tokens / decode wall-clock as in eval/interactive_gen.py:71-85."""
+def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temperature=None, top_k=None,
+             callback=None):
+    """Decode max_new_tokens tokens after the prompt.  Returns (token ids, decode seconds, tokens
+    per second); throughput is max_new_tokens / decode wall-clock as in
+    eval/interactive_gen.py:71-85.  Greedy by default; with `temperature` (and optionally
+    `top_k`) tokens are sampled as the reference's generation script does (it uses 0.6 / 5).
+    `callback(token)` is called with every new (1, 1) token tensor as soon as it is queued -
+    the streaming hook of the interactive script; reading the value synchronises."""
     dev = prompt_ids.device
     n = prompt_ids.shape[1]
+    sampling = temperature is not None
+
+    def pick(lg):
+        if sampling:
+            return sample(lg, temperature, top_k)[0]
+        return lg[:, -1].argmax(-1, keepdim=True)
+
     logits = model(prompt_ids, torch.arange(n, device=dev))
-    tok = logits[:, -1].argmax(-1, keepdim=True)
+    tok = pick(logits)
     static_tok = tok.clone()
     static_pos = torch.tensor([n], device=dev)
     out = [tok.clone()]
+    if callback is not None:
+        callback(out[-1])
 
     def step():
+        # the random draw stays outside the captured graph: a replay would repeat it
         lg = model.decode_fused(static_tok, static_pos) if fused else model(static_tok, static_pos)
-        return lg[:, -1].argmax(-1, keepdim=True)
+        return lg if sampling else pick(lg)
 
     graph = None
     if use_graph:
@@ -346,9 +379,13 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True):
             nxt = static_next
         else:
             nxt = step()
+        if sampling:
+            nxt = pick(nxt)
         static_tok.copy_(nxt)
         static_pos.add_(1)
         out.append(nxt.clone())
+        if callback is not None:
+            callback(out[-1])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     return torch.cat(out, dim=1), dt, (max_new_tokens - 1) / dt

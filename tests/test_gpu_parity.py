@@ -396,6 +396,23 @@ def test_decode_attention(heads, kv_heads, pos):
     assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
 
 
+def test_generate_sampling_and_streaming():
+    """Sampled decoding through the captured step: top_k = 1 reproduces the greedy tokens, a
+    wider draw stays inside the vocabulary, and the streaming callback sees every token in order."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
+    ids = torch.randint(0, cfg.vocab, (1, 7), generator=torch.Generator().manual_seed(3)).cuda()
+    greedy, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 8)
+    seen = []
+    top1, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 8, temperature=0.6, top_k=1,
+                          callback=lambda t: seen.append(t))
+    assert torch.equal(top1, greedy)
+    assert len(seen) == 8 and torch.equal(torch.cat(seen, dim=1), top1)
+    torch.manual_seed(5)
+    drawn, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 8, temperature=0.6, top_k=5)
+    assert drawn.shape == (1, 8) and int(drawn.min()) >= 0 and int(drawn.max()) < cfg.vocab
+
+
 def test_fused_decode_step_matches_generic():
     # the 13-launch fused decode step against the module-by-module forward of the same model
     from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder

@@ -150,3 +150,29 @@ def test_quantiser_entry_points_raise():
         cb.pack_trellis(torch.zeros(1, 128, dtype=torch.int32))
     with pytest.raises(ValueError):
         BitshiftLinear(16, 16, 16, 5, 2, 9, 'quantlut_sym', has_kernel=True)
+
+
+def test_sampling_helpers_follow_the_generation_script():
+    """top-k restriction and the exponential-race draw of eval/interactive_gen.py:15-40."""
+    from qtip_amd.llama_decode import logits_to_probs, sample
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(2, 50, generator=g)
+    p = logits_to_probs(logits, temperature=0.6, top_k=5)
+    assert torch.allclose(p.sum(-1), torch.ones(2))
+    assert ((p > 0).sum(-1) == 5).all()
+    top = logits.topk(5).indices
+    assert all(set(torch.nonzero(p[i]).flatten().tolist()) == set(top[i].tolist()) for i in range(2))
+    # ratios inside the kept set are those of softmax(logits / T)
+    full = torch.softmax(logits / 0.6, -1)
+    i0, i1 = top[0, 0], top[0, 1]
+    assert abs(p[0, i0] / p[0, i1] - full[0, i0] / full[0, i1]) < 1e-4
+    # top_k = 1 is greedy whatever the random draw
+    torch.manual_seed(1)
+    tok, _ = sample(logits[:, None, :], temperature=0.6, top_k=1)
+    assert (tok.flatten() == logits.argmax(-1)).all()
+    # the exponential race draws from the distribution: frequencies of a 3-way distribution
+    torch.manual_seed(2)
+    lg = torch.log(torch.tensor([0.7, 0.2, 0.1])).repeat(6000, 1)[:, None, :]
+    tok, _ = sample(lg)
+    freq = torch.bincount(tok.flatten(), minlength=3).float() / 6000
+    assert (freq - torch.tensor([0.7, 0.2, 0.1])).abs().max() < 0.03
