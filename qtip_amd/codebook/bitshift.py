@@ -171,6 +171,8 @@ class bitshift_codebook(nn.Module):
 
 class BitshiftLinear(nn.Module):
 
+    max_rows = 65535  # rows per launch of the transform / GEMM kernels (grid limit)
+
     def __init__(self, td_x, td_y, L, K, V, tlut_bits, decode_mode, dtype=torch.float16, tlut=None,
                  has_kernel=False):
         super().__init__()
@@ -253,6 +255,12 @@ class BitshiftLinear(nn.Module):
         dev = input.device
         x = input.reshape(-1, n)
         bs = x.shape[0]
+        if bs == 0:
+            return input.new_empty(*input.shape[:-1], m)
+        if bs > self.max_rows:  # the launchers take at most 65535 rows: go through in slabs
+            outs = [self.forward(x[i:i + self.max_rows], trellis, SU, SV, had_left, had_right, K_left, K_right,
+                                 rcp, tp_rank, mode=mode, **kwargs) for i in range(0, bs, self.max_rows)]
+            return torch.cat(outs, dim=0).view(*input.shape[:-1], m)
 
         # ---- input transform: fp16(H_L^T (x * SU) / sqrt(n) / 32)
         fused_in = (rcp != 1 and SU.dtype == torch.float16 and x.dtype in (torch.float16, torch.float32))

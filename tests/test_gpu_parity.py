@@ -490,6 +490,29 @@ def test_matvec_with_transform_in_prologue(K, m, k, S):
     assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()
 
 
+def test_forward_empty_and_slabbed_batches():
+    """No rows in, no rows out; more rows than one launch takes go through in slabs with the
+    same result as one pass."""
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    m, k, K = 256, 512, 3
+    L = make_layer(m, k, K, seed=4)
+    mod = BitshiftLinear(16, 16, 16, K, 2, 9, "quantlut_sym", tlut=dev(L["tlut"]), has_kernel=True)
+    hl, Kl = mh.get_hadK(k)
+    hr, Kr = mh.get_hadK(m)
+    args = (dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), hl, hr, Kl, Kr, 0, 8)
+    empty = mod(torch.empty(0, k, dtype=torch.float16, device="cuda"), *args)
+    assert empty.shape == (0, m) and empty.dtype == torch.float16
+    empty3 = mod(torch.empty(2, 0, k, dtype=torch.float16, device="cuda"), *args)
+    assert empty3.shape == (2, 0, m)
+    x = torch.randn(2, 5, k, generator=torch.Generator().manual_seed(1)).half().cuda()
+    whole = mod(x, *args)
+    mod.max_rows = 4  # 10 rows -> slabs of 4, 4, 2 (the last two through other kernels than the first)
+    slabbed = mod(x, *args)
+    assert slabbed.shape == whole.shape == (2, 5, m)
+    assert (slabbed.float() - whole.float()).abs().max() <= 2e-3 * whole.float().abs().max()
+
+
 @pytest.mark.parametrize("rcp", [1, 2])
 @pytest.mark.parametrize("bs", [1, 3])
 def test_forward_with_per_shard_transforms(rcp, bs):
