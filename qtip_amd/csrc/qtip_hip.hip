@@ -344,9 +344,19 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     matvec_accumulate<K>(ld, xv, slot4, acc);
   };
   int parity = 0, c_j = 0, c_rb = rb0;
+  int prio_phase = wave >> 2;  // waves w, w + 4, w + 8, w + 12 share a SIMD
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
+      // The hardware serves the waves of a SIMD oldest first, so the oldest finishes its share of a
+      // unit long before the youngest and the SIMD ends every unit on too few waves to hide
+      // latencies: the top issue priority rotates through the four waves, item by item.
+      switch ((prio_phase++) & 3) {
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+      }
       if (t + d < T) {
         if (c_j < nvj) {
           if constexpr (XLDS) {
@@ -730,15 +740,15 @@ hipError_t setup_once() {
     QTIP_ALLOW((decode_kernel<2>), kLutBytes)
     QTIP_ALLOW((decode_kernel<3>), kLutBytes)
     QTIP_ALLOW((decode_kernel<4>), kLutBytes)
-    QTIP_ALLOW((matvec_kernel<2, 4, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<3, 3, false>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<2, 2, false>), kMatvecLds)
+    QTIP_ALLOW((matvec_kernel<3, 2, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<2, 6, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 4, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 3, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 6, true, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 4, true, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 3, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
@@ -864,9 +874,9 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
     const size_t lds = kMatvecLds + (size_t)k * 2;
     auto* sg = (const uint16_t*)su_f16;
     switch (bits) {
-      case 2: matvec_kernel<2, 6, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
-      case 3: matvec_kernel<3, 4, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
-      default: matvec_kernel<4, 3, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      case 2: matvec_kernel<2, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      case 3: matvec_kernel<3, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      default: matvec_kernel<4, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
     }
     return (int)hipGetLastError();
   }
@@ -874,14 +884,14 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {
-      case 2: matvec_kernel<2, 6, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      case 3: matvec_kernel<3, 4, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      default: matvec_kernel<4, 3, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 3: matvec_kernel<3, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      default: matvec_kernel<4, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
     }
   } else {
     switch (bits) {
-      case 2: matvec_kernel<2, 4, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      case 3: matvec_kernel<3, 3, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 3: matvec_kernel<3, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
       default: matvec_kernel<4, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
     }
   }
