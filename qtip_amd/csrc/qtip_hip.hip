@@ -510,10 +510,16 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
       l_grp += gstep;
     }
   };
+  // table words first (their loads return before the stream's), one stage of the stream before the
+  // table is built, the others once the workgroup is past its first barrier
+  constexpr int NTW = kLutEntries * 4 / THREADS;  // distinct table words per thread
+  uint32_t tw[NTW];
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) issue(d);
+  for (int j = 0; j < NTW; ++j) tw[j] = tlut[j * (THREADS / 8) + (tid >> 3)];
+  issue(0);
 
   // ---- activation tiles: thread fills NB 16-byte chunks per tile
+
   static_assert(DEPTH % 2 == 0, "stage parity must be static inside the unrolled loop");
   u32x4 xg[2][NB];  // tiles on their way: [parity of the stage][chunk]
   auto load_tile = [&](int slot, int t) {  // stage t of a unit -> registers
@@ -538,9 +544,17 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
   };
   load_tile(0, 0);
   load_tile(1, nst > 1 ? 1 : 0);
-  build_lut128(lut, tlut, tid, THREADS);
+#pragma unroll
+  for (int it = 0; it < kLutEntries * 8 / THREADS; ++it) {
+    // item it*THREADS + tid belongs to entry it*THREADS/8 + tid/8; entries e and e+512 share a word
+    const uint32_t w = tw[it % NTW] ^ ((uint32_t)(it / NTW) << 15);
+    const u32x4 v = {w, w, w, w};
+    reinterpret_cast<u32x4*>(lut)[it * THREADS + tid] = v;
+  }
   store_tile(0, 0);
   __syncthreads();
+#pragma unroll
+  for (int d = 1; d < DEPTH; ++d) issue(d);
 
   float4_t acc[2][2][2][NB];  // [mh][rh][column half][batch tile]
 #pragma unroll
