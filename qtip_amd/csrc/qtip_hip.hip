@@ -344,6 +344,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     matvec_accumulate<K>(ld, xv, slot4, acc);
   };
   int parity = 0, c_j = 0, c_rb = rb0;
+  const uint32_t odd_mask = 0u - (uint32_t)(a & 1);
   int prio_phase = wave >> 2;  // waves w, w + 4, w + 8, w + 12 share a SIMD
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
@@ -390,8 +391,11 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           // element a % 2 holds the lane's sum over the four blocks; add the other column half
-          float v = (a & 1) ? acc[i][1] : acc[i][0];
+          // (bit select: a ternary on the two elements becomes a four-way dynamic extract)
+          const uint32_t e0 = __builtin_bit_cast(uint32_t, acc[i][0]), e1 = __builtin_bit_cast(uint32_t, acc[i][1]);
+          float v = __builtin_bit_cast(float, (e0 & ~odd_mask) | (e1 & odd_mask));
           v += dpp_xor1(v);
+
           acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
           if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
         }
