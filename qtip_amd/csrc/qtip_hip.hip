@@ -344,7 +344,6 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     matvec_accumulate<K>(ld, xv, slot4, acc);
   };
   int parity = 0, c_j = 0, c_rb = rb0;
-  const uint32_t odd_mask = 0u - (uint32_t)(a & 1);
   int prio_phase = wave >> 2;  // waves w, w + 4, w + 8, w + 12 share a SIMD
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
@@ -390,12 +389,11 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
         float* pp = part + parity * (kWaves * 32);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          // element a % 2 holds the lane's sum over the four blocks; add the other column half
-          // (bit select: a ternary on the two elements becomes a four-way dynamic extract)
-          const uint32_t e0 = __builtin_bit_cast(uint32_t, acc[i][0]), e1 = __builtin_bit_cast(uint32_t, acc[i][1]);
-          float v = __builtin_bit_cast(float, (e0 & ~odd_mask) | (e1 & odd_mask));
-          v += dpp_xor1(v);
-
+          // element a % 2 holds the lane's sum over the four blocks: an even lane adds its element 0
+          // and element 1 of its odd neighbour (the other column half).  Written without a
+          // per-lane choice of the element on purpose: with `v = odd ? e1 : e0; v += exchange(v)`
+          // the compiler, knowing that only even lanes store, fed e0 into the exchange for every lane.
+          const float v = acc[i][0] + dpp_xor1(acc[i][1]);
           acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
           if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
         }
@@ -649,9 +647,9 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
               for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                  float v = (a & 1) ? acc[mh][rh][1][nb][i] : acc[mh][rh][0][nb][i];
-                  v += dpp_xor1(v);
-                  vals[mh][rh][nb][i] = v;
+                  // even lanes: own sum of the even columns + the odd neighbour's sum of the odd columns
+                  // (no per-lane choice before the exchange, see matvec_kernel)
+                  vals[mh][rh][nb][i] = acc[mh][rh][0][nb][i] + dpp_xor1(acc[mh][rh][1][nb][i]);
                   acc[mh][rh][0][nb][i] = 0.f;
                   acc[mh][rh][1][nb][i] = 0.f;
                 }
