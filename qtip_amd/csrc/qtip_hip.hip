@@ -190,7 +190,7 @@ __device__ __forceinline__ void xform_prologue(const float v_in[8], float scale,
 // dst[s*m + 32*rb ...]: the result itself when S == 1, else one of S partial
 // vectors that the consumer adds in order (deterministic either way).
 //
-// The launcher makes gridDim.x a multiple of S: a workgroup keeps one k range
+// The launcher's grid is (S, workgroups per k range): a workgroup keeps one k range
 // [wl0, wl1) and walks row blocks rb0, rb0 + rb_step, ...  A wave sees its work
 // as a flat sequence of items (unit i, j) with wave-load wl0 + wave + 16*j;
 // every unit has npw items per wave of which the first nvj are real (the same
@@ -204,7 +204,7 @@ __device__ __forceinline__ void xform_prologue(const float v_in[8], float scale,
 template <int K, int DEPTH, bool XLDS, bool XFORM = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int S, int wl_per,
+    const uint32_t* __restrict__ tlut, int m, int k, int wl_per, int upw_q, int upw_r,
     const uint16_t* __restrict__ su = nullptr, float xscale = 1.f) {
   static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
   constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
@@ -225,14 +225,15 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const uint32_t loff = (uint32_t)lane * 8 * K;                // lane's bytes inside a wave-load
   const uint32_t xoff = (uint32_t)(32 * g + 4 * (a & 1)) * 2;  // lane's x bytes inside a wave-load
 
-  const int s = blockIdx.x % S;
-  const int rb0 = blockIdx.x / S;
-  const int rb_step = gridDim.x / S;
+  // grid = (S, workgroups per k range): no integer division on the way to the first loads
+  const int s = blockIdx.x;
+  const int rb0 = blockIdx.y;
+  const int rb_step = gridDim.y;
   const int wl0 = s * wl_per;
   const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
   const int wl1f = wl1 < nfull ? wl1 : nfull;           // end of the full wave-loads
   const int npw = (wl_per + kWaves - 1) / kWaves;       // items per wave and unit (padded)
-  const int upw = (nrb - rb0 + rb_step - 1) / rb_step;  // units of this workgroup
+  const int upw = upw_q + (rb0 < upw_r ? 1 : 0);  // units of this workgroup: ceil((nrb - rb0) / rb_step), quotient and remainder from the host
   const int T = upw * npw;
   const int w_first = wl0 + wave;
   const int nvj = w_first < wl1f ? (wl1f - w_first + kWaves - 1) / kWaves : 0;  // real items per unit
@@ -276,8 +277,19 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   // and 4 before are in between.)
   static_assert(kLutEntries * 8 == 8 * kThreads, "table build assumes 8 16-byte items per thread");
   uint32_t tw[4];  // item it*1024 + tid belongs to entry it*128 + tid/8; entries e and e+512 share a word
+  // the wave's eight words of a pass come through the scalar cache (uniform address), which
+  // keeps them out of the vector-memory queue that the stream requests fill
 #pragma unroll
-  for (int it = 0; it < 4; ++it) tw[it] = tlut[it * 128 + (tid >> 3)];
+  for (int it = 0; it < 4; ++it) {
+    const uint32_t* tp = tlut + it * 128 + wave * 8;
+    uint32_t sw[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sw[j] = tp[j];
+    uint32_t v = sw[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) v = ((lane >> 3) == j) ? sw[j] : v;
+    tw[it] = v;
+  }
   u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
   float xraw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if constexpr (XFORM) {
@@ -885,14 +897,17 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   auto* p = (const uint8_t*)packed;
   auto* xx = (const uint16_t*)x_f16;
   auto* t = (const uint32_t*)tlut;
+  const int per_range = (int)(grid / S);  // workgroups per k range, each walks row blocks rb0, rb0 + per_range, ...
+  const dim3 g2((unsigned)S, (unsigned)per_range);
+  const int uq = (m >> 5) / per_range, ur = (m >> 5) % per_range;
   if (su_f16) {
     // input transform inside the prologue: the whole transformed vector lives in LDS
     const size_t lds = kMatvecLds + (size_t)k * 2;
     auto* sg = (const uint16_t*)su_f16;
     switch (bits) {
-      case 2: matvec_kernel<2, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
-      case 3: matvec_kernel<3, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
-      default: matvec_kernel<4, 2, true, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per, sg, xscale); break;
+      case 2: matvec_kernel<2, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
+      case 3: matvec_kernel<3, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
+      default: matvec_kernel<4, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
     }
     return (int)hipGetLastError();
   }
@@ -900,15 +915,15 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {
-      case 2: matvec_kernel<2, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      case 3: matvec_kernel<3, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      default: matvec_kernel<4, 2, true><<<(int)grid, kThreads, lds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      case 3: matvec_kernel<3, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      default: matvec_kernel<4, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
     }
   } else {
     switch (bits) {
-      case 2: matvec_kernel<2, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      case 3: matvec_kernel<3, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
-      default: matvec_kernel<4, 2, false><<<(int)grid, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, S, wl_per); break;
+      case 2: matvec_kernel<2, 2, false><<<g2, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      case 3: matvec_kernel<3, 2, false><<<g2, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      default: matvec_kernel<4, 2, false><<<g2, kThreads, kMatvecLds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
     }
   }
   return (int)hipGetLastError();
