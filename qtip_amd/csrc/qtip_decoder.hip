@@ -40,7 +40,8 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   float* acc = red + 32;                         // [TG][D] partial outputs, TG*D = 8192
   float* p_s = acc + 8192;                       // [max_len] scores / probabilities
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int h = blockIdx.x, rep = H / Hkv, kvh = h / rep;
+  // grid = (query heads per kv head, kv heads): no integer division on the way to the loads
+  const int rep = gridDim.x, kvh = blockIdx.y, h = kvh * rep + blockIdx.x;
   const int pos = (int)pos_ptr[0];
   constexpr int half = D >> 1;
   const _Float16* q_in = qkv + (size_t)h * D;
@@ -52,8 +53,13 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   // ---- rotary embedding in fp16 arithmetic: x*cos + rotate_half(x)*sin
   if (tid < D) {
     const int i = tid < half ? tid : tid - half;
+    // the angle is the fp32 product the reference forms; its reduction to a fraction of a turn is
+    // done in fp64 (exact to 2^-29 of a turn at position 4096), the hardware cos / sin take turns.
+    // (cosf / sinf with their large-argument paths cost ~0.5 us on this kernel's critical path.)
     const float ang = (float)pos * inv_freq[i];
-    const _Float16 c = (_Float16)cosf(ang), s = (_Float16)sinf(ang);
+    const double turns = (double)ang * 0.15915494309189535;
+    const float fr = (float)(turns - __builtin_floor(turns));
+    const _Float16 c = (_Float16)__builtin_amdgcn_cosf(fr), s = (_Float16)__builtin_amdgcn_sinf(fr);
     const _Float16 q0 = q_in[tid], k0 = k_in[tid];
     const _Float16 qr = tid < half ? (_Float16)(-(float)q_in[tid + half]) : q_in[tid - half];
     const _Float16 kr = tid < half ? (_Float16)(-(float)k_in[tid + half]) : k_in[tid - half];
@@ -62,7 +68,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     q_s[tid] = (float)qe;
     k_s[tid] = (float)ke;
     v_s[tid] = (float)v_in[tid];
-    if (h % rep == 0 && pos < max_len) {
+    if (blockIdx.x == 0 && pos < max_len) {
       kc[(size_t)pos * D + tid] = ke;
       vc[(size_t)pos * D + tid] = v_in[tid];
     }
@@ -194,7 +200,7 @@ extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k
     return QTIP_E_SHAPE;
   const size_t lds = (size_t)(3 * kMaxHeadDim + 32 + 8192 + max_len) * sizeof(float);
 #define QTIP_ATTN(DD)                                                                               \
-  decode_attn_kernel<DD><<<heads, kAttnThreads, lds, (hipStream_t)stream>>>(                          \
+  decode_attn_kernel<DD><<<dim3((unsigned)(heads / kv_heads), (unsigned)kv_heads), kAttnThreads, lds, (hipStream_t)stream>>>(                          \
       (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,  \
       (const long*)pos_i64, inv_freq, heads, kv_heads, max_len)
   switch (head_dim) {

@@ -43,6 +43,10 @@ struct RhtParams {
   size_t in_row_stride;      // elements between consecutive rows of `in`
   float scale, eps;
   int in_parts, n, order, logA, pp, pre_mode;
+  // from the host (divisions and search loops in the prologue of a latency-bound kernel are time on
+  // its critical path): log2 of the column groups (vectorised form) or of the columns (scalar form),
+  // log2 of the waves holding a row in the transform, passes over the vector
+  int lcg, logw, npass;
 };
 
 template <typename T>
@@ -74,15 +78,15 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
   const int n = P.n, pp = P.pp, order = P.order;
   const TIn* src = reinterpret_cast<const TIn*>(P.in) + r * P.in_row_stride;
   const int OT = order << P.logA;
-  const int C = pp < kRhtThreads ? pp : kRhtThreads;  // pp <= kRhtThreads (launcher)
-  const int JG = kRhtThreads / C;
-  const int c = tid % C, jg = tid / C;
+  const int logc = P.lcg;              // log2(pp), pp <= kRhtThreads (launcher)
+  const int JG = kRhtThreads >> logc;
+  const int c = tid & (pp - 1), jg = tid >> logc;
   const int pre_mode = FUSED ? P.pre_mode : PRE_NONE;
 
   float z[RI];
 #pragma unroll
   for (int ri = 0; ri < RI; ++ri) z[ri] = 0.f;
-  const int npass = ((OT + JG - 1) / JG + CH - 1) / CH;  // the same for every thread (barriers inside)
+  const int npass = P.npass;  // the same for every thread (barriers inside)
   for (int pass = 0; pass < npass; ++pass) {
     const int j0 = jg + pass * JG * CH;
     // ---- all loads of this pass: elements j = j0, j0+JG, ... of column c.
@@ -176,21 +180,21 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
     __syncthreads();
   }
   // ---- thread t < RI*pp takes row t / pp, column t % pp
-  const int row = tid / pp, col = tid - row * pp;  // col keeps the lane index in its low bits
+  const int row = tid >> logc, col = tid & (pp - 1);  // col keeps the lane index in its low bits
   const bool active = tid < RI * pp;
   float y = 0.f;
   if (active) {
     if (JG > 1) {
-      for (int q = 0; q < JG; ++q) y += red[row][q * C + col];
+      for (int q = 0; q < JG; ++q) y += red[row][q * pp + col];
     } else {
       y = z[0];  // JG == 1 implies pp == 1024 and RI == 1
     }
   }
   if (JG > 1) __syncthreads();
   // ---- pp-point transform
-  const int W = pp > 64 ? pp >> 6 : 1;  // waves holding one row
-  int nb0 = 0;
-  while (nb0 < 6 && (1 << nb0) < pp) ++nb0;
+  const int logw = P.logw;
+  const int W = 1 << logw;  // waves holding one row
+  const int nb0 = logc < 6 ? logc : 6;
   int cfin = col;
   if (active) {
     y = wht_lanes(y, nb0, lane);
@@ -202,12 +206,10 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
       // transposed read: the wave index of the element becomes the low lane bits
       const int wv = col >> 6;
       const int ew = lane & (W - 1);              // wave part of the element index
-      const int el = (lane / W) + (64 / W) * wv;  // lane part of the element index
+      const int el = (lane >> logw) + (64 >> logw) * wv;  // lane part of the element index
       cfin = 64 * ew + el;
       y = red[row][cfin];
-      int nb = 0;
-      while ((1 << nb) < W) ++nb;
-      y = wht_lanes(y, nb, lane);
+      y = wht_lanes(y, logw, lane);
     }
   }
   if (active) {
@@ -277,20 +279,22 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   const int n = P.n, pp = P.pp, order = P.order;
   const TIn* src = reinterpret_cast<const TIn*>(P.in) + r * P.in_row_stride;
   const int OT = order << P.logA;
-  const int CG = pp >> 3;            // column groups of 8 (power of two, 1 .. 128)
-  const int JG = kRhtThreads / CG;   // row groups
-  int lcg = 0;
-  while ((1 << lcg) < CG) ++lcg;
+  // (logarithms and the pass count come from the host: divisions and search loops in the
+  // prologue of a latency-bound kernel are time on its critical path)
+  const int lcg = P.lcg;
+  const int CG = 1 << lcg;             // column groups of 8 (power of two, 1 .. 128)
+  const int JG = kRhtThreads >> lcg;   // row groups
   const int cg = tid & (CG - 1), jg = tid >> lcg;
   const int pre_mode = FUSED ? P.pre_mode : PRE_NONE;
 
   // ---- this thread's output element and its operands
   const bool active = tid < pp;
-  const int W = pp > 64 ? pp >> 6 : 1;  // waves holding the row in the transform
+  const int logw = P.logw;
+  const int W = 1 << logw;  // waves holding the row in the transform
   int cfin = tid;
   if (W > 1) {
     const int wv = tid >> 6;
-    cfin = 64 * (lane & (W - 1)) + (lane / W) + (64 / W) * wv;  // after the transposed read
+    cfin = 64 * (lane & (W - 1)) + (lane >> logw) + (64 >> logw) * wv;  // after the transposed read
   }
   const size_t oidx = ((size_t)iK * A + iA) * pp + cfin;
   float postv = 1.f, resv = 0.f;
@@ -302,7 +306,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   float z[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) z[e] = 0.f;
-  const int npass = ((OT + JG - 1) / JG + CH - 1) / CH;  // the same for every thread (barriers inside)
+  const int npass = P.npass;  // the same for every thread (barriers inside)
   for (int pass = 0; pass < npass; ++pass) {
     const int j0 = jg + pass * JG * CH;
     Raw8<TIn> xr[CH], ar[FUSED ? CH : 1];
@@ -433,8 +437,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   }
   __syncthreads();
   // ---- pp-point transform of column tid
-  int nb0 = 0;
-  while (nb0 < 6 && (1 << nb0) < pp) ++nb0;
+  const int nb0 = lcg + 3 < 6 ? lcg + 3 : 6;  // log2(pp), at most the six lane bits
   if (active) {
     y = wht_lanes(y, nb0, lane);
     if (W > 1) red[tid] = y;
@@ -443,9 +446,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
     __syncthreads();
     if (active) {
       y = red[cfin];
-      int nb = 0;
-      while ((1 << nb) < W) ++nb;
-      y = wht_lanes(y, nb, lane);
+      y = wht_lanes(y, logw, lane);
     }
   }
   if (active) {
@@ -460,9 +461,12 @@ template <typename TI, typename TO, bool FUSED>
 int launch_rht_vec(const RhtParams& P, dim3 grid, long loads, hipStream_t st) {
   // a prologue needs the whole row in one pass
   if (FUSED && P.pre_mode == PRE_RMSNORM && loads > 4) return QTIP_E_SHAPE;
-  if (loads <= 1) rht_vec_kernel<TI, TO, 1, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
-  else if (loads <= 2) rht_vec_kernel<TI, TO, 2, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
-  else rht_vec_kernel<TI, TO, 4, FUSED><<<grid, kRhtThreads, 0, st>>>(P);
+  const int ch = loads <= 1 ? 1 : loads <= 2 ? 2 : 4;
+  RhtParams Q = P;
+  Q.npass = (int)((loads + ch - 1) / ch);
+  if (loads <= 1) rht_vec_kernel<TI, TO, 1, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
+  else if (loads <= 2) rht_vec_kernel<TI, TO, 2, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
+  else rht_vec_kernel<TI, TO, 4, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
   return (int)hipGetLastError();
 }
 
@@ -470,13 +474,16 @@ template <typename TI, typename TO, bool FUSED>
 int launch_rht_l(const RhtParams& P, dim3 grid, long loads, int ri, hipStream_t st) {
   // a prologue needs the whole row in one pass
   if (FUSED && P.pre_mode == PRE_RMSNORM && loads > 16) return QTIP_E_SHAPE;
+  const int ch = ri == 4 ? (loads <= 8 ? 8 : 16) : (loads <= 4 ? 4 : loads <= 8 ? 8 : 16);
+  RhtParams Q = P;
+  Q.npass = (int)((loads + ch - 1) / ch);
   if (ri == 4) {
-    if (loads <= 8) rht_kernel<TI, TO, 8, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(P);
-    else rht_kernel<TI, TO, 16, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(P);
+    if (ch == 8) rht_kernel<TI, TO, 8, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(Q);
+    else rht_kernel<TI, TO, 16, FUSED, 4><<<grid, kRhtThreads, 0, st>>>(Q);
   } else {
-    if (loads <= 4) rht_kernel<TI, TO, 4, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
-    else if (loads <= 8) rht_kernel<TI, TO, 8, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
-    else rht_kernel<TI, TO, 16, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(P);
+    if (ch == 4) rht_kernel<TI, TO, 4, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(Q);
+    else if (ch == 8) rht_kernel<TI, TO, 8, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(Q);
+    else rht_kernel<TI, TO, 16, FUSED, 1><<<grid, kRhtThreads, 0, st>>>(Q);
   }
   return (int)hipGetLastError();
 }
@@ -520,6 +527,11 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
                       (!P.norm_w || (reinterpret_cast<uintptr_t>(P.norm_w) & 15u) == 0) &&
                       !(P.pre_mode == PRE_SILU_MUL && ((size_t)n * esz & 15u));
   if (vec_ok) {
+    int lcg = 0, logw = 0;
+    while ((8 << lcg) < pp) ++lcg;
+    while ((64 << logw) < pp) ++logw;
+    P.lcg = lcg;
+    P.logw = logw;
     const int JGv = kRhtThreads / (pp >> 3);
     const long vloads = (OT + JGv - 1) / JGv;
     dim3 vgrid((unsigned)OT, rows);
@@ -531,6 +543,13 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
     if (in_dtype == QTIP_F16 && out_dtype == QTIP_F32) return launch_rht_vec<_Float16, float, false>(P, vgrid, vloads, st);
     if (in_dtype == QTIP_F32 && out_dtype == QTIP_F16) return launch_rht_vec<float, _Float16, false>(P, vgrid, vloads, st);
     return launch_rht_vec<float, float, false>(P, vgrid, vloads, st);
+  }
+  {
+    int logc = 0, logw = 0;
+    while ((1 << logc) < pp) ++logc;
+    while ((64 << logw) < pp) ++logw;
+    P.lcg = logc;
+    P.logw = logw;
   }
   const int JG = kRhtThreads / pp;
   const long loads = (OT + JG - 1) / JG;
