@@ -162,7 +162,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
 #pragma unroll
       for (int q = 0; q < CH; ++q) {
         const float g = v[q];
-        const float sl = (float)(_Float16)(g / (1.f + __expf(-g)));
+        const float sl = (float)(_Float16)(g * __builtin_amdgcn_rcpf(1.f + __expf(-g)));
         v[q] = (float)(_Float16)(sl * aux[q]);
       }
     }
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float g = v[q][e];
-          const float sl = (float)(_Float16)(g / (1.f + __expf(-g)));
+          const float sl = (float)(_Float16)(g * __builtin_amdgcn_rcpf(1.f + __expf(-g)));
           v[q][e] = (float)(_Float16)(sl * up[e]);
         }
       }
