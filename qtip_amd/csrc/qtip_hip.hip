@@ -474,7 +474,8 @@ constexpr size_t kGemmLds = kLut128Bytes + 2 * kGemmTileBytes;
 template <int K, int NB, int DEPTH, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16, int S, int wl_per) {
+    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16, int wl_per, int upw_q,
+    int upw_r) {
   constexpr int THREADS = WAVES * 64;
   constexpr int KS = WAVES / kGemmRB;          // wave-loads per stage
   constexpr int ROWB = KS * 256;               // bytes per tile row
@@ -500,12 +501,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
 
-  const int s = blockIdx.x % S;
-  const int g0 = blockIdx.x / S, gstep = gridDim.x / S;
+  // grid = (S, workgroups per k range); unit counts as quotient and remainder from the host:
+  // no integer division on the way to the first loads
+  const int s = blockIdx.x;
+  const int g0 = blockIdx.y, gstep = gridDim.y;
   const int wl0 = s * wl_per;                                   // wl_per is a multiple of KS
   const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
   const int nst = wl1 > wl0 ? (wl1 - wl0 + KS - 1) / KS : 0;    // stages (KS wave-loads each) per unit
-  const int upw = g0 < ngroups ? (ngroups - g0 + gstep - 1) / gstep : 0;  // units of this workgroup
+  const int upw = upw_q + (g0 < upw_r ? 1 : 0);  // units of this workgroup: ceil((ngroups - g0) / gstep)
   const int T = upw * nst;
   float* out_s = dst + (size_t)s * batch * m;
 
@@ -529,7 +532,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
   constexpr int NTW = kLutEntries * 4 / THREADS;  // distinct table words per thread
   uint32_t tw[NTW];
 #pragma unroll
-  for (int j = 0; j < NTW; ++j) tw[j] = tlut[j * (THREADS / 8) + (tid >> 3)];
+  for (int j = 0; j < NTW; ++j) {
+    // the wave's eight words of a pass through the scalar cache (uniform address), lane l keeps word l / 8
+    const uint32_t* tp = tlut + j * (THREADS / 8) + wave * 8;
+    uint32_t v = tp[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) v = ((lane >> 3) == e) ? tp[e] : v;
+    tw[j] = v;
+  }
   issue(0);
 
   // ---- activation tiles: thread fills NB 16-byte chunks per tile
@@ -1036,13 +1046,15 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
     const long units = (long)ngroups * Sp;
     long grid = units < di.cus ? units : di.cus;
     grid -= grid % Sp;  // a workgroup keeps one k range
+    const int per_range = (int)(grid / Sp);
+    const dim3 g2((unsigned)Sp, (unsigned)per_range);
     float* o = out + (size_t)b0 * m;
     float* d = Sp > 1 ? (float*)workspace : o;
     const int rnd = Sp > 1 ? 0 : round_f16;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
 #define QTIP_GEMM(KB, NBT, WV)                                                                          \
-  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? (WV == 16 ? 2 : 4) : 2), WV><<<(int)grid, WV * 64, kGemmLds, st>>>( \
-      d, p, xx, t, m, k, nb, rnd, Sp, wl_per)
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? (WV == 16 ? 2 : 4) : 2), WV><<<g2, WV * 64, kGemmLds, st>>>( \
+      d, p, xx, t, m, k, nb, rnd, wl_per, ngroups / per_range, ngroups % per_range)
 #define QTIP_GEMM_K(KB)               \
   if (nb <= 16) QTIP_GEMM(KB, 1, 16); \
   else QTIP_GEMM(KB, 2, 8);
