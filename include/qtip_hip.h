@@ -98,6 +98,24 @@ int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const voi
                                      const void* su_f16, float scale, const void* tlut, int m, int k,
                                      int bits, int nparts, void* stream);
 
+/* qtip_decompress_matvec_parts with the whole boundary between two linear layers of a decoder
+ * in front of it (k in {2048, 4096, 8192}):
+ *   x_new = residual + fp16(scale_out * post * H_k (prev_parts[0] + prev_parts[1] + ...))
+ *   x_t   = fp16(scale_in * H_k (su * (norm_w * fp16(x_new * rsqrt(mean(x_new^2) + eps)))))
+ *   parts = hatW . x_t,   x_out = x_new
+ * i.e. the output transform of the previous QuantizedLinear (lib/codebook/bitshift.py:465-472) with
+ * the residual addition (model/llama.py:964,979), the RMSNorm (model/llama.py:129-135) and this
+ * layer's input transform (bitshift.py:428-441) and matvec in one launch: what qtip_rht_chain
+ * followed by qtip_decompress_matvec_parts computes.  prev_parts: prev_nparts vectors of k fp32,
+ * prev_part_stride floats apart; post fp32[k]; residual, norm_w, su fp16[k]; x_out fp16[k], not
+ * the residual buffer (every workgroup reads residual, one writes x_out); all 16-byte aligned. */
+int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const void* tlut, int m, int k,
+                                       int bits, int nparts, const float* prev_parts, int prev_nparts,
+                                       size_t prev_part_stride, const float* post, float scale_out,
+                                       const void* residual_f16, const void* norm_w_f16, float eps,
+                                       const void* su_f16, float scale_in, void* x_out_f16,
+                                       void* stream);
+
 /* Bytes of scratch qtip_decompress_gemm wants for this shape (0 when it does not split k). */
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch);
 

@@ -183,6 +183,108 @@ __device__ __forceinline__ void xform_prologue(const float v_in[8], float scale,
   __syncthreads();  // scratch is free for the table, xs is complete
 }
 
+// XFORM == 2: the whole boundary between two linear layers of a decoder in front of the matvec,
+//   x_new = residual + fp16(scale_out * post * H_k (sum of the previous layer's partial results)),
+//   x_t   = fp16(scale_in * H_k (su * RMSNorm(x_new) * norm_w)),    parts_out = hatW . x_t
+// i.e. the output transform of the previous QuantizedLinear with the residual addition, the
+// RMSNorm and the input transform of this one (what rht_chain_kernel does in a launch of its
+// own).  Every workgroup recomputes the k-point boundary - a few microseconds of work on 1024
+// threads, most of it while the first stream requests are in flight - and workgroup (0, 0)
+// stores x_new for the layers that follow.
+struct ChainArgs {
+  const float* parts;        // [in_parts][k] fp32 partial results of the previous linear layer
+  const float* post;         // its output sign vector times its scale (SV), k fp32
+  const _Float16* residual;  // the residual stream, k fp16
+  const _Float16* norm_w;    // RMSNorm weight, k fp16
+  _Float16* x_out;           // the new residual stream, k fp16
+  size_t part_stride;        // floats between partial results
+  float scale_out, eps;
+  int in_parts;
+};
+struct ChainRegs {  // a thread's operands, k / 1024 <= 8 consecutive elements each
+  float v[8], pv[8], rv[8], wv[8], sv[8];
+};
+
+template <int EPT>
+__device__ __forceinline__ void chain_load(const ChainArgs& c, const _Float16* su, int tid, int lane,
+                                           int wave, ChainRegs& r) {
+  using namespace qtip_wht;
+  const int e_nat = tid * EPT;
+  const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
+  // operands of the middle part in the swapped layout, the partial results in the natural one
+  ld_f32<EPT>(c.post + e_swp, r.pv);
+  ld_f16<EPT>(c.residual + e_swp, r.rv);
+  ld_f16<EPT>(c.norm_w + e_swp, r.wv);
+  ld_f16<EPT>(su + e_swp, r.sv);
+  ld_f32<EPT>(c.parts + e_nat, r.v);
+  for (int w = 1; w < c.in_parts; ++w) {
+    float t[EPT];
+    ld_f32<EPT>(c.parts + w * c.part_stride + e_nat, t);
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) r.v[i] += t[i];
+  }
+}
+
+// xbuf: k + k/64 floats of exchange buffer, wsum: 16 floats, xs: the k fp16 activations of the matvec
+template <int EPT>
+__device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, float scale_in, float* xbuf,
+                                              float* wsum, _Float16* xs, int tid, int lane, int wave,
+                                              bool write_x) {
+  using namespace qtip_wht;
+  constexpr int N = kThreads * EPT;
+  const int e_nat = tid * EPT;
+  const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
+  float v[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = r.v[i];
+  // ---- first transform (natural -> swapped layout)
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_nat + i)] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(xbuf[xidx<EPT>(e_swp + i)], 4, lane);
+  // ---- residual, RMSNorm, sign vector of this layer
+  float ss = 0.f;
+  _Float16 xn[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    const float o = v[i] * c.scale_out * r.pv[i];
+    xn[i] = (_Float16)(r.rv[i] + (float)(_Float16)o);
+    v[i] = (float)xn[i];
+    ss += v[i] * v[i];
+  }
+  if (write_x) st_f16<EPT>(c.x_out + e_swp, xn);
+  ss = wave_sum(ss);
+  if (lane == 0) wsum[wave] = ss;
+  __syncthreads();  // also: every read of xbuf above is done
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) tot += wsum[w];
+  const float rs = __builtin_amdgcn_rsqf(tot / (float)N + c.eps);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = (float)(_Float16)(r.wv[i] * (float)(_Float16)(v[i] * rs)) * r.sv[i];
+  // ---- second transform (swapped -> natural layout)
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_swp + i)] = v[i];
+  __syncthreads();
+  // the bits still missing are the top four of the element's lane field = lane bits 2..5 here
+  _Float16 xo[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    float y = xbuf[xidx<EPT>(e_nat + i)];
+    y = wht_lanes(y, 6, lane, 2);
+    xo[i] = (_Float16)(y * scale_in);
+  }
+  st_f16<EPT>(xs + e_nat, xo);
+  __syncthreads();  // the exchange buffer is free for the table, xs is complete
+}
+
 // Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup take
 // the unit's wave-loads round-robin (so the workgroup streams one contiguous
 // run of bytes), reduce across the four blocks of a wave-load inside the MFMA, across the two
@@ -201,11 +303,13 @@ __device__ __forceinline__ void xform_prologue(const float v_in[8], float scale,
 // access) and are skipped by the arithmetic.
 // XLDS: the x values of the workgroup's k range are staged in LDS once
 // (needs 256 bytes per wave-load of the range) and read from there.
-template <int K, int DEPTH, bool XLDS, bool XFORM = false>
+// XFORM: 0 = x is the matvec's fp16 input, 1 = x is the layer's raw input (input transform in the
+// prologue), 2 = the previous layer's partial results (whole layer boundary in the prologue).
+template <int K, int DEPTH, bool XLDS, int XFORM = 0>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
     const uint32_t* __restrict__ tlut, int m, int k, int wl_per, int upw_q, int upw_r,
-    const uint16_t* __restrict__ su = nullptr, float xscale = 1.f) {
+    const uint16_t* __restrict__ su = nullptr, float xscale = 1.f, const ChainArgs chain = ChainArgs{}) {
   static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
   constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
   extern __shared__ __align__(16) uint8_t smem[];
@@ -292,7 +396,15 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   }
   u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
   float xraw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if constexpr (XFORM) {
+  ChainRegs cr;
+  if constexpr (XFORM == 2) {
+    const _Float16* sr = reinterpret_cast<const _Float16*>(su);
+    switch (k >> 10) {
+      case 2: chain_load<2>(chain, sr, tid, lane, wave, cr); break;
+      case 4: chain_load<4>(chain, sr, tid, lane, wave, cr); break;
+      default: chain_load<8>(chain, sr, tid, lane, wave, cr); break;
+    }
+  } else if constexpr (XFORM == 1) {
     // the raw activations and the sign vector of the layer, k / 1024 consecutive elements per thread
     using namespace qtip_wht;
     float sv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -319,7 +431,17 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
   for (int d = 0; d < FIRST; ++d) issue(d);
 
-  if constexpr (XFORM) {
+  if constexpr (XFORM == 2) {
+    float* xbuf = reinterpret_cast<float*>(smem);
+    float* wsum = xbuf + k + (k >> 6);
+    _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
+    const bool write_x = blockIdx.x == 0 && blockIdx.y == 0;
+    switch (k >> 10) {
+      case 2: chain_compute<2>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
+      case 4: chain_compute<4>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
+      default: chain_compute<8>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
+    }
+  } else if constexpr (XFORM == 1) {
     float* scratch = reinterpret_cast<float*>(smem);
     _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
     switch (k >> 10) {
@@ -784,9 +906,12 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, 2>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, 2>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, 2>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
     QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
@@ -841,7 +966,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 7; }
+int qtip_abi_version(void) { return 8; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -897,7 +1022,7 @@ size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
 
 static int launch_matvec(float* dst, const void* packed, const void* x_f16, const void* tlut, int m,
                          int k, int bits, int S, hipStream_t st, const void* su_f16 = nullptr,
-                         float xscale = 1.f) {
+                         float xscale = 1.f, const ChainArgs* chain = nullptr) {
   DeviceInfo& di = device_info();
   const long units = (long)(m >> 5) * S;
   long grid = units < di.cus ? units : di.cus;
@@ -914,10 +1039,18 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
     // input transform inside the prologue: the whole transformed vector lives in LDS
     const size_t lds = kMatvecLds + (size_t)k * 2;
     auto* sg = (const uint16_t*)su_f16;
+    if (chain) {
+      switch (bits) {
+        case 2: matvec_kernel<2, 2, true, 2><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale, *chain); break;
+        case 3: matvec_kernel<3, 2, true, 2><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale, *chain); break;
+        default: matvec_kernel<4, 2, true, 2><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale, *chain); break;
+      }
+      return (int)hipGetLastError();
+    }
     switch (bits) {
-      case 2: matvec_kernel<2, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
-      case 3: matvec_kernel<3, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
-      default: matvec_kernel<4, 2, true, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
+      case 2: matvec_kernel<2, 2, true, 1><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
+      case 3: matvec_kernel<3, 2, true, 1><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
+      default: matvec_kernel<4, 2, true, 1><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur, sg, xscale); break;
     }
     return (int)hipGetLastError();
   }
@@ -970,6 +1103,34 @@ int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const voi
   if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
   if (!aligned16(x_raw_f16) || !aligned16(su_f16)) return QTIP_E_ALIGN;
   return launch_matvec(parts, packed, x_raw_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale);
+}
+
+int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const void* tlut, int m, int k,
+                                       int bits, int nparts, const float* prev_parts, int prev_nparts,
+                                       size_t prev_part_stride, const float* post, float scale_out,
+                                       const void* residual_f16, const void* norm_w_f16, float eps,
+                                       const void* su_f16, float scale_in, void* x_out_f16,
+                                       void* stream) {
+  int rc = check_matvec(parts, packed, su_f16, tlut, m, k, bits);
+  if (rc) return rc;
+  if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
+  if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
+  if (prev_nparts < 1 || prev_nparts > kMaxSplit || x_out_f16 == residual_f16) return QTIP_E_SHAPE;
+  if (!aligned16(prev_parts) || !aligned16(post) || !aligned16(residual_f16) || !aligned16(norm_w_f16) ||
+      !aligned16(su_f16) || !aligned16(x_out_f16) || ((prev_part_stride * sizeof(float)) & 15u))
+    return QTIP_E_ALIGN;
+  ChainArgs c;
+  c.parts = prev_parts;
+  c.post = post;
+  c.residual = (const _Float16*)residual_f16;
+  c.norm_w = (const _Float16*)norm_w_f16;
+  c.x_out = (_Float16*)x_out_f16;
+  c.part_stride = prev_part_stride;
+  c.scale_out = scale_out;
+  c.eps = eps;
+  c.in_parts = prev_nparts;
+  return launch_matvec(parts, packed, su_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale_in, &c);
 }
 
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,

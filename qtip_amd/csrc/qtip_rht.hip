@@ -650,11 +650,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_chain_kernel(
 #pragma unroll
   for (int i = 0; i < EPT; ++i) {
     float y = xbuf[xidx<EPT>(e_nat + i)];
-#pragma unroll
-    for (int b = 2; b < 6; ++b) {
-      const float o = lane_xor(y, b);
-      y = ((lane >> b) & 1) ? o - y : y + o;
-    }
+    y = wht_lanes(y, 6, lane, 2);
     xo[i] = (_Float16)(y * scale_in);
   }
   st_f16<EPT>(xt_out + row * N + e_nat, xo);

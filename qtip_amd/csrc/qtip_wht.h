@@ -31,10 +31,10 @@ __device__ __forceinline__ float lane_xor(float v, int b) {
 }
 
 // Walsh-Hadamard butterflies over lane bits 0 .. nbits-1 (natural order)
-__device__ __forceinline__ float wht_lanes(float v, int nbits, int lane) {
+__device__ __forceinline__ float wht_lanes(float v, int nbits, int lane, int lo = 0) {
 #pragma unroll
   for (int b = 0; b < 6; ++b) {
-    if (b < nbits) {
+    if (b >= lo && b < nbits) {
       const float o = lane_xor(v, b);
       v = ((lane >> b) & 1) ? o - v : v + o;
     }

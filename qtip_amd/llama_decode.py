@@ -138,20 +138,21 @@ class DecoderLayer(nn.Module):
             self._fused = {n: _FusedLinear(getattr(self, n)) for n in names}
         return self._fused
 
-    def decode_fused(self, x, k_cache, v_cache, pos, inv_freq, xt_qkv=None, next_layer=None):
+    def decode_fused(self, x, k_cache, v_cache, pos, inv_freq, qkv_parts=None, next_layer=None):
         """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
         layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections.
         With power-of-two hidden sizes the [transform-out + residual] of o / down and the
         [RMSNorm + transform-in] that follows are one launch and the o projection transforms its
-        input inside the matvec (10 per layer): `xt_qkv` is then the
-        already transformed input of this layer's qkv matvec (made by the previous layer) and
-        `next_layer` the layer whose qkv input this one prepares.  Returns (x, xt for the next layer)."""
+        input inside the matvec (10 per layer); where it pays, that one launch is the following
+        matvec itself (8 per layer): `qkv_parts` are then the partial sums of this layer's qkv matvec
+        (launched by the previous layer with the layer boundary in its prologue) and `next_layer` the
+        layer whose qkv matvec this one launches.  Returns (x, qkv partial sums for the next layer)."""
         cfg = self.cfg
         f = self._fused_linears()
         if self.fused:
-            if xt_qkv is None:
-                xt_qkv = f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
-            qkv = f['qkv'].transform_out(f['qkv'].matvec(xt_qkv))
+            if qkv_parts is None:
+                qkv_parts = f['qkv'].matvec(f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps))
+            qkv = f['qkv'].transform_out(qkv_parts)
         else:
             qkv = torch.cat([f[n](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
                              for n in ('q_proj', 'k_proj', 'v_proj')], dim=-1)
@@ -159,8 +160,8 @@ class DecoderLayer(nn.Module):
                                     cfg.head_dim)
         if self.fused and f['o'].can_chain_into(f['up_gate']):
             parts = f['o'].matvec_from(attn.reshape(1, -1))
-            x, xt_ug = f['o'].chain(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
-            ug = f['up_gate'].transform_out(f['up_gate'].matvec(xt_ug))
+            x, ug_parts = f['o'].chain_matvec(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
+            ug = f['up_gate'].transform_out(ug_parts)
         else:
             x = f['o'](attn.reshape(1, -1), residual=x)
             if self.fused:
@@ -171,7 +172,7 @@ class DecoderLayer(nn.Module):
         nq = next_layer._fused_linears().get('qkv') if (next_layer is not None and next_layer.fused) else None
         if nq is not None and not f['down'].dense and f['down'].can_chain_into(nq):
             parts = f['down'].matvec(f['down'].transform_in(ug, ops.PRE_SILU_MUL))
-            return f['down'].chain(parts, x, nq, next_layer.input_norm.weight, cfg.eps)
+            return f['down'].chain_matvec(parts, x, nq, next_layer.input_norm.weight, cfg.eps)
         return f['down'](ug, ops.PRE_SILU_MUL, residual=x), None
 
 
@@ -240,6 +241,19 @@ class _FusedLinear:
         return ops.rht_chain(parts, self.SV, (self.m**-0.5) * 32.0, residual, norm_weight, eps, nxt.SU,
                              (nxt.n**-0.5) / 32.0)
 
+    def chain_matvec(self, parts, residual, nxt, norm_weight, eps):
+        """(x_new, partial sums of nxt's matvec) from this layer's partial sums: the layer boundary
+        runs inside nxt's matvec launch where that is faster than a launch of its own (measured:
+        always for 4096-long vectors; for 8192 only in front of the smaller matrices, since every
+        workgroup of the matvec repeats the boundary), else chain + matvec."""
+        if nxt.n <= 4096 or nxt.m <= 16384:
+            p, x_new = ops.decompress_matvec_parts_chain(nxt.trellis, nxt.tlut, nxt.m, nxt.n, nxt.K, parts, self.SV,
+                                                         (self.m**-0.5) * 32.0, residual, norm_weight, eps, nxt.SU,
+                                                         (nxt.n**-0.5) / 32.0)
+            return x_new, p.unsqueeze(1)
+        x_new, xt = self.chain(parts, residual, nxt, norm_weight, eps)
+        return x_new, nxt.matvec(xt)
+
     def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
         if self.dense:
             return self._dense(x, pre_mode, norm_weight, eps, residual)
@@ -302,10 +316,10 @@ class LlamaDecoder(nn.Module):
     def decode_fused(self, tok, pos):
         """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab) fp32, fused kernels."""
         x = self.embed[tok.reshape(-1)]
-        xt = None
+        qp = None
         for i, layer in enumerate(self.layers):
             nxt = self.layers[i + 1] if i + 1 < len(self.layers) else None
-            x, xt = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq, xt, nxt)
+            x, qp = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq, qp, nxt)
         x = self.norm(x)
         return (x @ self.lm_head.T).float().reshape(1, 1, -1)
 

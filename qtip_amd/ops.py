@@ -142,6 +142,37 @@ def decompress_matvec_parts_rht(packed, x_raw, su, scale, tlut, m, k, bits, npar
     return parts
 
 
+def decompress_matvec_parts_chain(packed, tlut, m, k, bits, prev_parts, post, scale_out, residual, norm_weight, eps,
+                                  su, scale_in, nparts=None):
+    """(parts, x_new): the boundary between two linear layers and the second layer's matvec in
+    one launch - x_new = fp16(residual + fp16(post * scale_out * H(sum(prev_parts)))),
+    parts = decode(packed) @ fp16(scale_in * H(su * rmsnorm(x_new))), the (S, m) fp32 partial sums.
+    prev_parts: (S_prev, k) or (S_prev, 1, k) fp32; k in RHT_IN_MATVEC_SIZES."""
+    _check_packed(packed, m, k, bits)
+    _check_tlut(tlut, packed.device)
+    require_cuda(prev_parts, "prev_parts", torch.float32)
+    require_cuda(post, "post", torch.float32)
+    require_cuda(residual, "residual", torch.float16)
+    require_cuda(norm_weight, "norm_weight", torch.float16)
+    require_cuda(su, "su", torch.float16)
+    pp = prev_parts.reshape(prev_parts.shape[0], -1)
+    if k not in RHT_IN_MATVEC_SIZES or pp.shape[1] != k:
+        raise ValueError(f"prev_parts must hold vectors of k = {k} values, k in {RHT_IN_MATVEC_SIZES}")
+    if any(t.numel() != k for t in (post, residual, norm_weight, su)):
+        raise ValueError(f"post, residual, norm_weight and su must hold k = {k} values")
+    if any(t.device != packed.device for t in (pp, post, residual, norm_weight, su)):
+        raise ValueError(f"all operands must be on {packed.device}")
+    S = int(nparts) if nparts is not None else matvec_split(m, k, bits, packed.device)
+    parts = torch.empty((S, m), dtype=torch.float32, device=packed.device)
+    x_new = torch.empty((1, k), dtype=torch.float16, device=packed.device)
+    with torch.cuda.device(packed.device):
+        check(lib().qtip_decompress_matvec_parts_chain(
+            _ptr(parts), _ptr(packed), _ptr(tlut), m, k, bits, S, _ptr(pp), pp.shape[0], ctypes.c_size_t(pp.stride(0)),
+            _ptr(post), ctypes.c_float(scale_out), _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), _ptr(su),
+            ctypes.c_float(scale_in), _ptr(x_new), stream_ptr(packed.device)), "qtip_decompress_matvec_parts_chain")
+    return parts, x_new
+
+
 def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     """(batch, m) fp32 = x[batch,k] (fp16) @ decode(packed)[m,k]^T on the matrix cores."""
     _check_packed(packed, m, k, bits)

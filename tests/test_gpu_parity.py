@@ -396,6 +396,25 @@ def test_decode_attention(heads, kv_heads, pos):
     assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
 
 
+def test_fused_decode_with_layer_boundaries_in_the_matvec():
+    """Hidden size 2048: the o -> up/gate and down -> next qkv boundaries run inside the following
+    matvec launch (8 launches per layer); same logits and caches as the module-by-module forward."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder
+    cfg = LlamaConfig(hidden=2048, heads=16, kv_heads=16, layers=3, ffn=172 * 16, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64)
+    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(5, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([5], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        b = model.decode_fused(tok, pos)
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    for c0, c1 in zip(kc, model.k_cache):
+        assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+
+
 def test_generate_sampling_and_streaming():
     """Sampled decoding through the captured step: top_k = 1 reproduces the greedy tokens, a
     wider draw stays inside the vocabulary, and the streaming callback sees every token in order."""
@@ -511,6 +530,31 @@ def test_forward_empty_and_slabbed_batches():
     slabbed = mod(x, *args)
     assert slabbed.shape == whole.shape == (2, 5, m)
     assert (slabbed.float() - whole.float()).abs().max() <= 2e-3 * whole.float().abs().max()
+
+
+@pytest.mark.parametrize("K", [2, 4])
+@pytest.mark.parametrize("m,k,S,Sp", [(256, 2048, None, 1), (1024, 4096, 1, 2), (4096, 4096, None, 2), (512, 8192, 4, 1),
+                                      (2048, 8192, None, 3)])
+def test_matvec_with_layer_boundary_in_prologue(K, m, k, S, Sp):
+    """[output transform + residual + RMSNorm + input transform] inside the matvec launch against
+    the chained-transform launch followed by the plain matvec: same residual stream bit for bit
+    (same arithmetic in the same order), partial sums to rounding."""
+    from qtip_amd import ops
+    L = make_layer(m, k, K, seed=m + k + K + 1)
+    g = torch.Generator().manual_seed(K + m + Sp)
+    prev = torch.randn(Sp, 1, k, generator=g).cuda()
+    SV = (torch.sign(torch.randn(k, generator=g)) * (0.5 + torch.rand(k, generator=g))).cuda()
+    res = torch.randn(1, k, generator=g).half().cuda()
+    w = (1 + 0.1 * torch.randn(k, generator=g)).half().cuda()
+    su = dev(L["SU"]).half()
+    so, si, eps = 32.0 * k**-0.5, k**-0.5 / 32.0, 1e-5
+    packed, tlut = dev(L["packed"]).reshape(-1), dev(L["tlut"]).reshape(-1)
+    parts, x_new = ops.decompress_matvec_parts_chain(packed, tlut, m, k, K, prev, SV, so, res, w, eps, su, si, nparts=S)
+    x_ref, xt_ref = ops.rht_chain(prev, SV, so, res, w, eps, su, si)
+    ref = ops.decompress_matvec_parts(packed, xt_ref.reshape(-1), tlut, m, k, K, nparts=S)
+    assert torch.equal(x_new, x_ref)
+    assert parts.shape == ref.shape
+    assert torch.equal(parts, ref)
 
 
 @pytest.mark.parametrize("rcp", [1, 2])
