@@ -192,6 +192,22 @@ int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
                           const void* pos_i64, const float* inv_freq, int heads, int kv_heads,
                           int head_dim, int max_len, void* stream);
 
+/* qtip_decode_attention on the qkv projection's raw matvec result: the output transform of
+ * BitshiftLinear.forward (lib/codebook/bitshift.py:465-472: H_R, then * SV * 32) runs in the
+ * kernel's prologue, each workgroup producing the three head-sized slices it needs, so the
+ * [q | k | v] vector never exists in memory and the transform is no launch of its own.
+ *   qkv = post * scale * (H_order (x) H_{n/order}) (parts[0] + ... + parts[in_parts-1]),
+ * n = (heads + 2 kv_heads) * head_dim, n / order a power of two >= head_dim; had_bits = the packed
+ * sign bits of the order x order table as qtip_rht takes them (NULL when order == 1); parts 16-byte
+ * aligned fp32, part_stride (elements) a multiple of 4; head_dim 64 or 128.  Values are rounded to
+ * fp16 where the layer's output is (the transform's sums are taken in another order than
+ * qtip_rht's, so results agree to fp32 rounding before that cast, not bit for bit). */
+int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, size_t part_stride,
+                              const float* post_f32, float scale, const uint32_t* had_bits, int order,
+                              void* k_cache_f16, void* v_cache_f16, const void* pos_i64,
+                              const float* inv_freq, int heads, int kv_heads, int head_dim, int max_len,
+                              void* stream);
+
 /* ---- packing tools (natural packing = one circular big-endian bitstream per tile, stored as
  * T*K/16 little-endian uint16 words; state i is the 16-bit window at bit i*K*V) ---------------- */
 

@@ -7,6 +7,7 @@
 #include <stdint.h>
 
 #include "../../include/qtip_hip.h"
+#include "qtip_wht.h"
 
 namespace {
 
@@ -24,14 +25,32 @@ __device__ __forceinline__ float wave_reduce_sum(float v) {
   return v;
 }
 
+// The qkv projection's output transform, for the XF form of the kernel: the new token's
+// [q | k | v] vector (n = order * 2^logp2 elements) is
+//   post * scale * (H_order (x) H_{2^logp2}) (sum of the in_parts partial sums),
+// and a workgroup needs three D-long slices of it.  A slice (table row iK, block b of the
+// power-of-two part) is the D-point Walsh-Hadamard transform of
+//   u[c] = sum_{jK, b'} (-1)^(bits[jK][iK] + popcount(b & b')) v[(jK * 2^logp2) + b' * D + c],
+// n additions per slice instead of a launch of its own for the whole vector.
+struct AttnXf {
+  const float* parts;
+  const float* post;
+  const uint32_t* had_bits;
+  size_t part_stride;
+  float scale;
+  int in_parts, order, logp2, n;
+};
+
+typedef float float4a __attribute__((ext_vector_type(4)));
+
 // One workgroup per query head.  qkv: [H*D | Hkv*D | Hkv*D] fp16 of the new
 // token; k_cache / v_cache: [Hkv][max_len][D] fp16; pos_ptr: position of the
 // new token (device memory, so that a recorded graph follows the position).
-template <int D>
+template <int D, bool XF>
 __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     _Float16* __restrict__ out, const _Float16* __restrict__ qkv, _Float16* __restrict__ k_cache,
     _Float16* __restrict__ v_cache, const long* __restrict__ pos_ptr,
-    const float* __restrict__ inv_freq, int H, int Hkv, int max_len) {
+    const float* __restrict__ inv_freq, int H, int Hkv, int max_len, const AttnXf X) {
   extern __shared__ __align__(16) uint8_t smem[];
   float* q_s = reinterpret_cast<float*>(smem);   // [D] rotated query (as fp16 values)
   float* k_s = q_s + kMaxHeadDim;                // [D] rotated new key
@@ -50,27 +69,154 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   _Float16* kc = k_cache + (size_t)kvh * max_len * D;
   _Float16* vc = v_cache + (size_t)kvh * max_len * D;
 
-  // ---- rotary embedding in fp16 arithmetic: x*cos + rotate_half(x)*sin
+  // rotary angle of this thread's dimension, requested before anything else: the angle is the fp32
+  // product the reference forms; its reduction to a fraction of a turn is done in fp64 (exact to
+  // 2^-29 of a turn at position 4096), the hardware cos / sin take turns.  (cosf / sinf with their
+  // large-argument paths cost ~0.5 us on this kernel's critical path.)
+  _Float16 rc = (_Float16)1.f, rs = (_Float16)0.f;
   if (tid < D) {
-    const int i = tid < half ? tid : tid - half;
-    // the angle is the fp32 product the reference forms; its reduction to a fraction of a turn is
-    // done in fp64 (exact to 2^-29 of a turn at position 4096), the hardware cos / sin take turns.
-    // (cosf / sinf with their large-argument paths cost ~0.5 us on this kernel's critical path.)
-    const float ang = (float)pos * inv_freq[i];
+    const float ang = (float)pos * inv_freq[tid < half ? tid : tid - half];
     const double turns = (double)ang * 0.15915494309189535;
     const float fr = (float)(turns - __builtin_floor(turns));
-    const _Float16 c = (_Float16)__builtin_amdgcn_cosf(fr), s = (_Float16)__builtin_amdgcn_sinf(fr);
-    const _Float16 q0 = q_in[tid], k0 = k_in[tid];
-    const _Float16 qr = tid < half ? (_Float16)(-(float)q_in[tid + half]) : q_in[tid - half];
-    const _Float16 kr = tid < half ? (_Float16)(-(float)k_in[tid + half]) : k_in[tid - half];
+    rc = (_Float16)__builtin_amdgcn_cosf(fr);
+    rs = (_Float16)__builtin_amdgcn_sinf(fr);
+  }
+
+  if constexpr (XF) {
+    static_assert(D == 64 || D == 128, "the transform prologue holds 3 x 16 x D partial sums in LDS");
+    constexpr int LOGD = D == 64 ? 6 : 7;
+    constexpr int G = D / 4, R = kAttnThreads / G;  // float4 column groups, chunk rows per pass
+    constexpr int QP = 4, WP = 2;                   // chunk rows and partial sums in flight per thread
+    const int g = tid & (G - 1), r = tid >> (LOGD - 2);
+    const int logb = X.logp2 - LOGD, bmask = (1 << logb) - 1;
+    const int nrows = X.n >> LOGD;
+    // slices: q of head h, k and v of its kv head
+    const int off[3] = {h * D, (H + kvh) * D, (H + Hkv + kvh) * D};
+    int iK[3], bb[3];
+#pragma unroll
+    for (int s3 = 0; s3 < 3; ++s3) {
+      iK[s3] = off[s3] >> X.logp2;
+      bb[s3] = (off[s3] >> LOGD) & bmask;
+    }
+    // the epilogue's operand, requested with everything else
+    const int s3 = tid >> LOGD, c = tid & (D - 1);
+    float postv = 1.f;
+    if (tid < 3 * D && X.post) postv = X.post[off[s3 < 3 ? s3 : 0] + c];
+    // table words: with order 1 the index is 0 and the word is masked out (any readable address does)
+    const uint32_t* hb = X.order > 1 ? X.had_bits : reinterpret_cast<const uint32_t*>(X.parts);
+    const uint32_t omask = X.order > 1 ? 1u : 0u;
+    float a[3][4];  // (plain arrays: element-wise bit operations on vector-typed values went wrong in the compiler)
+#pragma unroll
+    for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[s3][e] = 0.f;
+    for (int j0 = 0; j0 < nrows; j0 += QP * R) {
+      float v[QP][4];
+      uint32_t hw[QP][3];
+#pragma unroll
+      for (int q = 0; q < QP; ++q) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[q][e] = 0.f;
+        const int j = j0 + r + q * R;
+        const int jc = j < nrows ? j : 0;
+#pragma unroll
+        for (int s3 = 0; s3 < 3; ++s3) {
+          const unsigned bit = (unsigned)(jc >> logb) * X.order + iK[s3];
+          hw[q][s3] = hb[bit >> 5] >> (bit & 31);
+        }
+      }
+      for (int w0 = 0; w0 < X.in_parts; w0 += WP) {
+        float4a raw[QP][WP];
+#pragma unroll
+        for (int u = 0; u < WP; ++u) {
+          if (w0 + u < X.in_parts) {
+#pragma unroll
+            for (int q = 0; q < QP; ++q) {
+              const int j = j0 + r + q * R;
+              const int jc = j < nrows ? j : 0;
+              raw[q][u] = *reinterpret_cast<const float4a*>(X.parts + (size_t)(w0 + u) * X.part_stride +
+                                                            ((size_t)jc << LOGD) + 4 * g);
+            }
+          } else {
+#pragma unroll
+            for (int q = 0; q < QP; ++q) raw[q][u] = float4a{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < WP; ++u)
+#pragma unroll
+          for (int q = 0; q < QP; ++q) {
+            v[q][0] += raw[q][u].x;
+            v[q][1] += raw[q][u].y;
+            v[q][2] += raw[q][u].z;
+            v[q][3] += raw[q][u].w;
+          }
+      }
+#pragma unroll
+      for (int q = 0; q < QP; ++q) {
+        const int j = j0 + r + q * R;
+        if (j < nrows) {
+#pragma unroll
+          for (int s3 = 0; s3 < 3; ++s3) {
+            const uint32_t sg = (((hw[q][s3] & omask) ^ (uint32_t)__builtin_popcount(bb[s3] & j & bmask)) & 1u) << 31;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              a[s3][e] += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[q][e]) ^ sg);
+          }
+        }
+      }
+    }
+    // rows that share a wave, then one partial slice per wave
+#pragma unroll
+    for (int o = 32; o >= G; o >>= 1)
+#pragma unroll
+      for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[s3][e] += __shfl_xor(a[s3][e], o);
+    if (lane < G) {
+#pragma unroll
+      for (int s3 = 0; s3 < 3; ++s3)
+        *reinterpret_cast<float4a*>(acc + (s3 * 16 + wave) * D + 4 * g) =
+            float4a{a[s3][0], a[s3][1], a[s3][2], a[s3][3]};
+    }
+    __syncthreads();
+    float y = 0.f;
+    if (tid < 3 * D) {
+#pragma unroll
+      for (int w = 0; w < 16; ++w) y += acc[(s3 * 16 + w) * D + c];
+      y = qtip_wht::wht_lanes(y, 6, lane);
+      if (D > 64) q_s[s3 * kMaxHeadDim + c] = y;
+    }
+    __syncthreads();  // the partial slices are consumed: their space takes the fp16 result
+    _Float16* h_s = reinterpret_cast<_Float16*>(acc);
+    if (tid < 3 * D) {
+      if (D > 64) {
+        const float other = q_s[s3 * kMaxHeadDim + (c ^ 64)];
+        y = (c & 64) ? other - y : y + other;
+      }
+      h_s[s3 * D + c] = (_Float16)(y * X.scale * postv);
+    }
+    __syncthreads();
+  }
+  const _Float16* h_s = reinterpret_cast<const _Float16*>(acc);
+  auto QV = [&](int i) -> _Float16 { return XF ? h_s[i] : q_in[i]; };
+  auto KV = [&](int i) -> _Float16 { return XF ? h_s[D + i] : k_in[i]; };
+  auto VV = [&](int i) -> _Float16 { return XF ? h_s[2 * D + i] : v_in[i]; };
+
+  // ---- rotary embedding in fp16 arithmetic: x*cos + rotate_half(x)*sin
+  if (tid < D) {
+    const _Float16 c = rc, s = rs;
+    const _Float16 q0 = QV(tid), k0 = KV(tid), v0 = VV(tid);
+    const _Float16 qr = tid < half ? (_Float16)(-(float)QV(tid + half)) : QV(tid - half);
+    const _Float16 kr = tid < half ? (_Float16)(-(float)KV(tid + half)) : KV(tid - half);
     const _Float16 qe = (_Float16)((float)(_Float16)((float)q0 * (float)c) + (float)(_Float16)((float)qr * (float)s));
     const _Float16 ke = (_Float16)((float)(_Float16)((float)k0 * (float)c) + (float)(_Float16)((float)kr * (float)s));
     q_s[tid] = (float)qe;
     k_s[tid] = (float)ke;
-    v_s[tid] = (float)v_in[tid];
+    v_s[tid] = (float)v0;
     if (blockIdx.x == 0 && pos < max_len) {
       kc[(size_t)pos * D + tid] = ke;
-      vc[(size_t)pos * D + tid] = v_in[tid];
+      vc[(size_t)pos * D + tid] = v0;
     }
   }
   __syncthreads();
@@ -191,23 +337,67 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
 
 }  // namespace
 
-extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
-                                     void* v_cache_f16, const void* pos_i64, const float* inv_freq,
-                                     int heads, int kv_heads, int head_dim, int max_len, void* stream) {
-  if (!out_f16 || !qkv_f16 || !k_cache_f16 || !v_cache_f16 || !pos_i64 || !inv_freq) return QTIP_E_NULL;
+static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf, void* k_cache_f16,
+                            void* v_cache_f16, const void* pos_i64, const float* inv_freq, int heads,
+                            int kv_heads, int head_dim, int max_len, void* stream) {
+  if (!out_f16 || !k_cache_f16 || !v_cache_f16 || !pos_i64 || !inv_freq) return QTIP_E_NULL;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads || head_dim < 64 || head_dim > kMaxHeadDim ||
       (head_dim & (head_dim - 1)) || max_len < 1 || max_len > 4096)
     return QTIP_E_SHAPE;
   const size_t lds = (size_t)(3 * kMaxHeadDim + 32 + 8192 + max_len) * sizeof(float);
-#define QTIP_ATTN(DD)                                                                               \
-  decode_attn_kernel<DD><<<dim3((unsigned)(heads / kv_heads), (unsigned)kv_heads), kAttnThreads, lds, (hipStream_t)stream>>>(                          \
+  const dim3 grid((unsigned)(heads / kv_heads), (unsigned)kv_heads);
+#define QTIP_ATTN(DD, XX, ARG)                                                                      \
+  decode_attn_kernel<DD, XX><<<grid, kAttnThreads, lds, (hipStream_t)stream>>>(                      \
       (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,  \
-      (const long*)pos_i64, inv_freq, heads, kv_heads, max_len)
-  switch (head_dim) {
-    case 64: QTIP_ATTN(64); break;
-    case 128: QTIP_ATTN(128); break;
-    default: QTIP_ATTN(256); break;
+      (const long*)pos_i64, inv_freq, heads, kv_heads, max_len, ARG)
+  if (xf) {
+    if (head_dim == 64) QTIP_ATTN(64, true, *xf);
+    else if (head_dim == 128) QTIP_ATTN(128, true, *xf);
+    else return QTIP_E_SHAPE;
+  } else {
+    switch (head_dim) {
+      case 64: QTIP_ATTN(64, false, AttnXf{}); break;
+      case 128: QTIP_ATTN(128, false, AttnXf{}); break;
+      default: QTIP_ATTN(256, false, AttnXf{}); break;
+    }
   }
 #undef QTIP_ATTN
   return (int)hipGetLastError();
+}
+
+extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
+                                     void* v_cache_f16, const void* pos_i64, const float* inv_freq,
+                                     int heads, int kv_heads, int head_dim, int max_len, void* stream) {
+  if (!qkv_f16) return QTIP_E_NULL;
+  return launch_attention(out_f16, qkv_f16, nullptr, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads,
+                          kv_heads, head_dim, max_len, stream);
+}
+
+extern "C" int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, size_t part_stride,
+                                         const float* post_f32, float scale, const uint32_t* had_bits,
+                                         int order, void* k_cache_f16, void* v_cache_f16,
+                                         const void* pos_i64, const float* inv_freq, int heads,
+                                         int kv_heads, int head_dim, int max_len, void* stream) {
+  if (!parts || (order > 1 && !had_bits)) return QTIP_E_NULL;
+  if (in_parts < 1 || in_parts > 16 || order < 1 || order > 256 || heads < 1 || kv_heads < 1 ||
+      head_dim < 64 || head_dim > 128)
+    return QTIP_E_SHAPE;
+  const long n = (long)(heads + 2 * kv_heads) * head_dim;
+  if (n % order) return QTIP_E_SHAPE;
+  const long p2 = n / order;
+  if ((p2 & (p2 - 1)) || p2 < head_dim || n > (1 << 20)) return QTIP_E_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(parts) & 15) || (part_stride & 3)) return QTIP_E_SHAPE;
+  AttnXf x;
+  x.parts = parts;
+  x.post = post_f32;
+  x.had_bits = had_bits;
+  x.part_stride = part_stride;
+  x.scale = scale;
+  x.in_parts = in_parts;
+  x.order = order;
+  x.logp2 = 0;
+  while ((1L << x.logp2) < p2) ++x.logp2;
+  x.n = (int)n;
+  return launch_attention(out_f16, nullptr, &x, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
+                          head_dim, max_len, stream);
 }

@@ -139,12 +139,13 @@ class DecoderLayer(nn.Module):
         return self._fused
 
     def decode_fused(self, x, k_cache, v_cache, pos, inv_freq, qkv_parts=None, next_layer=None):
-        """One new token, x (1, hidden) fp16, on the fused transforms: 13 launches for the fused
-        layout (4 x [transform, matvec, transform] + attention), 24 for the separate projections.
+        """One new token, x (1, hidden) fp16, on the fused transforms: 12 launches for the fused
+        layout (4 x [transform, matvec, transform] + attention, the attention kernel doing the qkv
+        output transform itself), 24 for the separate projections.
         With power-of-two hidden sizes the [transform-out + residual] of o / down and the
         [RMSNorm + transform-in] that follows are one launch and the o projection transforms its
-        input inside the matvec (10 per layer); where it pays, that one launch is the following
-        matvec itself (8 per layer): `qkv_parts` are then the partial sums of this layer's qkv matvec
+        input inside the matvec (9 per layer); where it pays, that one launch is the following
+        matvec itself (7 per layer): `qkv_parts` are then the partial sums of this layer's qkv matvec
         (launched by the previous layer with the layer boundary in its prologue) and `next_layer` the
         layer whose qkv matvec this one launches.  Returns (x, qkv partial sums for the next layer)."""
         cfg = self.cfg
@@ -152,12 +153,18 @@ class DecoderLayer(nn.Module):
         if self.fused:
             if qkv_parts is None:
                 qkv_parts = f['qkv'].matvec(f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps))
-            qkv = f['qkv'].transform_out(qkv_parts)
+            qkv = None if f['qkv'].out_transform_fits_attention(cfg.head_dim) else f['qkv'].transform_out(qkv_parts)
         else:
             qkv = torch.cat([f[n](x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps)
                              for n in ('q_proj', 'k_proj', 'v_proj')], dim=-1)
-        attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
-                                    cfg.head_dim)
+        if qkv is None:
+            # the attention kernel transforms the head-sized slices it needs itself
+            q = f['qkv']
+            attn = ops.decode_attention_rht(qkv_parts, q.SV, (q.m**-0.5) * 32.0, q.br, q.Kr, k_cache, v_cache, pos,
+                                            inv_freq, cfg.heads, cfg.kv_heads, cfg.head_dim)
+        else:
+            attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
+                                        cfg.head_dim)
         if self.fused and f['o'].can_chain_into(f['up_gate']):
             parts = f['o'].matvec_from(attn.reshape(1, -1))
             x, ug_parts = f['o'].chain_matvec(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
@@ -229,6 +236,13 @@ class _FusedLinear:
         return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
                        post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
                        residual=residual)
+
+    def out_transform_fits_attention(self, head_dim):
+        """The output transform can run in the attention kernel's prologue (head-sized slices of a
+        table-order x power-of-two transform)."""
+        p2 = self.m // self.Kr
+        return (not self.dense and head_dim in (64, 128) and p2 >= head_dim and p2 & (p2 - 1) == 0
+                and self.m <= 16384)
 
     def can_chain_into(self, nxt):
         """This layer's output transform and `nxt`'s input transform are plain power-of-two

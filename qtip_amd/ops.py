@@ -300,6 +300,38 @@ def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head
     return out
 
 
+def decode_attention_rht(parts, post, scale, had_bits, order, k_cache, v_cache, pos, inv_freq, heads, kv_heads,
+                         head_dim):
+    """decode_attention on the qkv projection's raw matvec result `parts` (S, n) fp32: the
+    projection's output transform (order x power-of-two Hadamard, * post * scale, cast to fp16) runs
+    in the attention kernel's prologue.  had_bits: the table's packed sign bits (None for order 1)."""
+    require_cuda(parts, "parts", torch.float32)
+    require_cuda(k_cache, "k_cache", torch.float16)
+    require_cuda(v_cache, "v_cache", torch.float16)
+    require_cuda(pos, "pos", torch.int64)
+    require_cuda(inv_freq, "inv_freq", torch.float32)
+    if post is not None:
+        require_cuda(post, "post", torch.float32)
+    if had_bits is not None:
+        require_cuda(had_bits, "had_bits", torch.int32)
+    n = (heads + 2 * kv_heads) * head_dim
+    parts = parts.reshape(-1, n)
+    max_len = k_cache.shape[-2]
+    if k_cache.numel() != kv_heads * max_len * head_dim or v_cache.shape != k_cache.shape \
+            or inv_freq.numel() != head_dim // 2 or pos.numel() != 1 or (post is not None and post.numel() != n) \
+            or (order > 1 and had_bits is None):
+        raise ValueError("decode_attention_rht: inconsistent shapes")
+    out = torch.empty(heads * head_dim, dtype=torch.float16, device=parts.device)
+    with torch.cuda.device(parts.device):
+        check(lib().qtip_decode_attention_rht(_ptr(out), _ptr(parts), parts.shape[0], parts.stride(0),
+                                              _ptr(post) if post is not None else None, float(scale),
+                                              _ptr(had_bits) if had_bits is not None else None, int(order),
+                                              _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), heads,
+                                              kv_heads, head_dim, max_len, stream_ptr(parts.device)),
+              "qtip_decode_attention_rht")
+    return out
+
+
 # ---- packing tools ---------------------------------------------------------------------------
 
 def repack(packed, m, k, bits, to_kernel=True):

@@ -396,6 +396,36 @@ def test_decode_attention(heads, kv_heads, pos):
     assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,D,S", [(32, 32, 128, 1), (64, 8, 128, 2), (8, 8, 128, 3), (16, 16, 64, 1),
+                                                 (4, 2, 128, 2), (4, 2, 64, 5), (56, 8, 128, 1)])
+def test_decode_attention_with_output_transform_in_prologue(heads, kv_heads, D, S):
+    """Attention on the qkv projection's raw partial sums == output transform (a launch of its
+    own, checked against the oracle elsewhere) followed by attention: the same fp16 q/k/v up to the
+    summation order of the transform, so caches and outputs agree to fp16 rounding."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits
+    n = (heads + 2 * kv_heads) * D
+    max_len, pos = 256, 77
+    g = torch.Generator().manual_seed(n + S)
+    parts = (torch.randn(S, n, generator=g) * 0.3).cuda()
+    post = (torch.sign(torch.randn(n, generator=g) + 1e-5) * (1.0 + 0.1 * torch.rand(n, generator=g))).cuda()
+    hadK, order = get_hadK(n)
+    bits = had_bits(hadK, order, False, "cuda") if order > 1 else None
+    scale = n**-0.5
+    kc = (torch.randn(1, kv_heads, max_len, D, generator=g) * 0.5).half().cuda()
+    vc = torch.randn(1, kv_heads, max_len, D, generator=g).half().cuda()
+    kc1, vc1 = kc.clone(), vc.clone()
+    inv_freq = (1.0 / (10000.0**(torch.arange(0, D, 2).float() / D))).cuda()
+    p = torch.tensor([pos], device="cuda")
+    qkv = ops.rht(parts if S > 1 else parts.reshape(1, n), order=order, had_bits=bits, post=post, scale=scale,
+                  out_dtype=torch.float16, in_parts=S)
+    ref = ops.decode_attention(qkv.reshape(-1), kc, vc, p, inv_freq, heads, kv_heads, D)
+    got = ops.decode_attention_rht(parts, post, scale, bits, order, kc1, vc1, p, inv_freq, heads, kv_heads, D)
+    assert torch.allclose(kc1.float(), kc.float(), atol=2e-3, rtol=2e-3)
+    assert torch.allclose(vc1.float(), vc.float(), atol=2e-3, rtol=2e-3)
+    assert_close(got.float().cpu().numpy(), ref.float().cpu().numpy(), 5e-3, 1e-3)
+
+
 def test_fused_decode_with_layer_boundaries_in_the_matvec():
     """Hidden size 2048: the o -> up/gate and down -> next qkv boundaries run inside the following
     matvec launch (8 launches per layer); same logits and caches as the module-by-module forward."""
