@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch over algorithmic bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this script, each calibrated against a 256 MiB copy (summary under profiles/)
-MEASURED_TRAFFIC_RATIO = {("70b", 2): (52550.0 + 82.0) / 52224.0}
+MEASURED_TRAFFIC_RATIO = {("70b", 2): (52582.0 + 82.0) / 52224.0}
 SHAPES_70B = [("qkv", 10240, 8192), ("o", 8192, 8192), ("up_gate", 57344, 8192), ("down", 8192, 28672)]
 SHAPES_7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("up_gate", 22016, 4096), ("down", 4096, 11008)]
 
