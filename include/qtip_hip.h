@@ -208,6 +208,18 @@ int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, s
                               const float* inv_freq, int heads, int kv_heads, int head_dim, int max_len,
                               void* stream);
 
+/* Final RMSNorm of the decoder for one vector: out = weight * fp16(x * rsqrt(mean(x^2) + eps))
+ * (model/llama.py:129-135), n <= 16384, one launch instead of the module's six. */
+int qtip_rmsnorm(void* out_f16, const void* x_f16, const void* weight_f16, float eps, int n, void* stream);
+
+/* Greedy token pick of the generation loop (eval/interactive_gen.py:43-69: argmax of the last
+ * position's logits, copy into the next step's input, position + 1), all in device memory so a
+ * recorded graph decodes token after token: tok_i64[0] = argmax(logits_f16[0..vocab)) (first index
+ * among equal maxima; NaNs never win), history_i64[pos - history_base] = that token when the slot
+ * lies in [0, history_len) (history may be NULL), pos_i64[0] += 1.  logits 16-byte aligned. */
+int qtip_greedy_pick(const void* logits_f16, int vocab, void* tok_i64, void* pos_i64, void* history_i64,
+                     long history_len, long history_base, void* stream);
+
 /* ---- packing tools (natural packing = one circular big-endian bitstream per tile, stored as
  * T*K/16 little-endian uint16 words; state i is the 16-bit window at bit i*K*V) ---------------- */
 

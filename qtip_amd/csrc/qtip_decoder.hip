@@ -401,3 +401,123 @@ extern "C" int qtip_decode_attention_rht(void* out_f16, const float* parts, int 
   return launch_attention(out_f16, nullptr, &x, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
                           head_dim, max_len, stream);
 }
+
+// ---- token head of the decode loop: final RMSNorm and the greedy pick ------------------------
+
+namespace {
+
+constexpr int kHeadThreads = 1024;
+
+// out = w * fp16(x * rsqrt(mean(x^2) + eps)) for one vector (model/llama.py:129-135), one workgroup
+__global__ __launch_bounds__(kHeadThreads) void rmsnorm_kernel(_Float16* __restrict__ out,
+                                                               const _Float16* __restrict__ x,
+                                                               const _Float16* __restrict__ w, float eps,
+                                                               int n) {
+  __shared__ float wsum[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int MAXE = 16;  // n <= 16384
+  float v[MAXE], g[MAXE];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < MAXE; ++e) {
+    const int i = tid + e * kHeadThreads;
+    v[e] = i < n ? (float)x[i] : 0.f;
+    g[e] = i < n ? (float)w[i] : 0.f;
+    ss += v[e] * v[e];
+  }
+  ss = qtip_wht::wave_sum(ss);
+  if (lane == 0) wsum[wave] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) tot += wsum[q];
+  const float rs = __builtin_amdgcn_rsqf(tot / (float)n + eps);
+#pragma unroll
+  for (int e = 0; e < MAXE; ++e) {
+    const int i = tid + e * kHeadThreads;
+    if (i < n) out[i] = (_Float16)(g[e] * (float)(_Float16)(v[e] * rs));
+  }
+}
+
+// argmax of fp16 logits (first index among equal maxima, NaNs never win), stored as the next
+// input token and into the history slot of this position; the position advances by one.  All in
+// device memory, so a recorded graph decodes token after token without host work in between
+// (eval/interactive_gen.py:43-69 does this with argmax, copies and an increment per token).
+__global__ __launch_bounds__(kHeadThreads) void greedy_pick_kernel(const _Float16* __restrict__ logits, int vocab,
+                                                                   long* __restrict__ tok, long* __restrict__ pos,
+                                                                   long* __restrict__ hist, long hist_len,
+                                                                   long hist_base) {
+  __shared__ float bv[16];
+  __shared__ int bi[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  const int nch = vocab >> 3;  // 16-byte chunks
+  for (int c = tid; c < nch; c += kHeadThreads) {
+    const uint4 raw = reinterpret_cast<const uint4*>(logits)[c];
+    const _Float16* h = reinterpret_cast<const _Float16*>(&raw);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)h[e];
+      if (f > best) {  // chunks come in increasing order per thread: the first maximum stays
+        best = f;
+        idx = c * 8 + e;
+      }
+    }
+  }
+  for (int i = (nch << 3) + tid; i < vocab; i += kHeadThreads) {
+    const float f = (float)logits[i];
+    if (f > best) {
+      best = f;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float ob = __shfl_xor(best, o);
+    const int oi = __shfl_xor(idx, o);
+    if (ob > best || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if (lane == 0) {
+    bv[wave] = best;
+    bi[wave] = idx;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int q = 1; q < 16; ++q)
+      if (bv[q] > best || (bv[q] == best && bi[q] < idx)) {
+        best = bv[q];
+        idx = bi[q];
+      }
+    if (idx == 0x7fffffff) idx = 0;  // nothing compared greater than -inf
+    const long p = pos[0];
+    const long slot = p - hist_base;
+    if (hist && slot >= 0 && slot < hist_len) hist[slot] = idx;
+    tok[0] = idx;
+    pos[0] = p + 1;
+  }
+}
+
+}  // namespace
+
+extern "C" int qtip_rmsnorm(void* out_f16, const void* x_f16, const void* weight_f16, float eps, int n,
+                            void* stream) {
+  if (!out_f16 || !x_f16 || !weight_f16) return QTIP_E_NULL;
+  if (n < 1 || n > 16 * kHeadThreads) return QTIP_E_SHAPE;
+  rmsnorm_kernel<<<1, kHeadThreads, 0, (hipStream_t)stream>>>((_Float16*)out_f16, (const _Float16*)x_f16,
+                                                             (const _Float16*)weight_f16, eps, n);
+  return (int)hipGetLastError();
+}
+
+extern "C" int qtip_greedy_pick(const void* logits_f16, int vocab, void* tok_i64, void* pos_i64,
+                                void* history_i64, long history_len, long history_base, void* stream) {
+  if (!logits_f16 || !tok_i64 || !pos_i64) return QTIP_E_NULL;
+  if (vocab < 1 || history_len < 0 || (reinterpret_cast<uintptr_t>(logits_f16) & 15)) return QTIP_E_SHAPE;
+  greedy_pick_kernel<<<1, kHeadThreads, 0, (hipStream_t)stream>>>((const _Float16*)logits_f16, vocab, (long*)tok_i64,
+                                                                 (long*)pos_i64, (long*)history_i64, history_len,
+                                                                 history_base);
+  return (int)hipGetLastError();
+}

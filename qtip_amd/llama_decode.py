@@ -327,15 +327,18 @@ class LlamaDecoder(nn.Module):
         x = self.norm(x)
         return (x @ self.lm_head.T).float()
 
-    def decode_fused(self, tok, pos):
-        """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab) fp32, fused kernels."""
+    def decode_fused(self, tok, pos, float_logits=True):
+        """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab), fused kernels;
+        fp32 as the reference returns them, or the fp16 values the lm_head product yields
+        (float_logits=False, what the greedy pick reads)."""
         x = self.embed[tok.reshape(-1)]
         qp = None
         for i, layer in enumerate(self.layers):
             nxt = self.layers[i + 1] if i + 1 < len(self.layers) else None
             x, qp = layer.decode_fused(x, self.k_cache[i], self.v_cache[i], pos, self.inv_freq, qp, nxt)
-        x = self.norm(x)
-        return (x @ self.lm_head.T).float().reshape(1, 1, -1)
+        x = ops.rmsnorm(x, self.norm.weight, self.norm.eps)
+        lg = (x @ self.lm_head.T).reshape(1, 1, -1)
+        return lg.float() if float_logits else lg
 
 
 def logits_to_probs(logits, temperature=1.0, top_k=None):
@@ -378,35 +381,58 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
     tok = pick(logits)
     static_tok = tok.clone()
     static_pos = torch.tensor([n], device=dev)
+    # greedy decoding on the fused kernels keeps its bookkeeping on the device: the pick kernel
+    # writes the next input token, the history slot and the advanced position, so a step is one
+    # graph replay and nothing else
+    on_device = fused and not sampling
+    history = torch.zeros(max(max_new_tokens, 1), dtype=torch.int64, device=dev)
+    history[0] = tok.reshape(-1)[0]
     out = [tok.clone()]
     if callback is not None:
         callback(out[-1])
 
     def step():
         # the random draw stays outside the captured graph: a replay would repeat it
+        if on_device:
+            lg = model.decode_fused(static_tok, static_pos, float_logits=False)
+            ops.greedy_pick(lg.reshape(-1), static_tok, static_pos, history, n - 1)
+            return None
         lg = model.decode_fused(static_tok, static_pos) if fused else model(static_tok, static_pos)
         return lg if sampling else pick(lg)
 
     graph = None
     if use_graph:
+        keep = (static_tok.clone(), static_pos.clone(), history.clone())
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
             for _ in range(2):
                 step()
+                if on_device:  # the warm-up steps must not advance the decode
+                    static_tok.copy_(keep[0])
+                    static_pos.copy_(keep[1])
+                    history.copy_(keep[2])
         torch.cuda.current_stream().wait_stream(s)
         # the warm-up wrote cache slot n with this token's k/v, which the timed step rewrites identically
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             static_next = step()
+        if on_device:  # capture only records; restore in case the stream ran anything
+            static_tok.copy_(keep[0])
+            static_pos.copy_(keep[1])
+            history.copy_(keep[2])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(max_new_tokens - 1):
+    for i in range(max_new_tokens - 1):
         if graph is not None:
             graph.replay()
             nxt = static_next
         else:
             nxt = step()
+        if on_device:
+            if callback is not None:
+                callback(history[i + 1:i + 2].view(1, 1))
+            continue
         if sampling:
             nxt = pick(nxt)
         static_tok.copy_(nxt)
@@ -416,4 +442,6 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
             callback(out[-1])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    if on_device:
+        return history[:max_new_tokens].view(1, -1).clone(), dt, (max_new_tokens - 1) / dt
     return torch.cat(out, dim=1), dt, (max_new_tokens - 1) / dt

@@ -332,6 +332,37 @@ def decode_attention_rht(parts, post, scale, had_bits, order, k_cache, v_cache, 
     return out
 
 
+def rmsnorm(x, weight, eps):
+    """weight * fp16(x * rsqrt(mean(x^2) + eps)) for one fp16 vector (model/llama.py:129-135)."""
+    require_cuda(x, "x", torch.float16)
+    require_cuda(weight, "weight", torch.float16)
+    if x.numel() != weight.numel():
+        raise ValueError("rmsnorm: x and weight differ in length")
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        check(lib().qtip_rmsnorm(_ptr(out), _ptr(x), _ptr(weight), float(eps), x.numel(), stream_ptr(x.device)),
+              "qtip_rmsnorm")
+    return out
+
+
+def greedy_pick(logits, tok, pos, history=None, history_base=0):
+    """tok[0] = argmax(logits) (fp16 logits of one position, first index among equal maxima),
+    history[pos - history_base] = tok when that slot exists, pos += 1 - the per-token bookkeeping
+    of a greedy generation loop (eval/interactive_gen.py:43-69) in one launch, in place."""
+    require_cuda(logits, "logits", torch.float16)
+    require_cuda(tok, "tok", torch.int64)
+    require_cuda(pos, "pos", torch.int64)
+    if history is not None:
+        require_cuda(history, "history", torch.int64)
+    if tok.numel() != 1 or pos.numel() != 1:
+        raise ValueError("greedy_pick: tok and pos hold one element each")
+    with torch.cuda.device(logits.device):
+        check(lib().qtip_greedy_pick(_ptr(logits), logits.numel(), _ptr(tok), _ptr(pos),
+                                     _ptr(history) if history is not None else None,
+                                     history.numel() if history is not None else 0, int(history_base),
+                                     stream_ptr(logits.device)), "qtip_greedy_pick")
+
+
 # ---- packing tools ---------------------------------------------------------------------------
 
 def repack(packed, m, k, bits, to_kernel=True):

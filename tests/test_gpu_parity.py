@@ -268,6 +268,20 @@ def test_errors_raise_not_exit():
         ops.decode(pk, tl[:100], 64, 64, 2)
     with pytest.raises(ValueError):
         ops.rht(torch.zeros(3, 100, device="cuda"))
+    # the launches with a transform in their prologue take a closed set of sizes
+    su = torch.ones(64, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.decompress_matvec_parts_rht(pk, x, su, 0.1, tl, 64, 64, 2)  # k not in {2048, 4096, 8192}
+    kc = torch.zeros(1, 2, 16, 256, dtype=torch.float16, device="cuda")
+    inv = torch.ones(128, device="cuda")
+    from qtip_amd._lib import QtipLibraryError
+    with pytest.raises(QtipLibraryError):  # head size 256 has no transform prologue (refused by the library)
+        ops.decode_attention_rht(torch.zeros(1, 8 * 256, device="cuda"), None, 1.0, None, 1, kc, kc.clone(),
+                                 torch.tensor([0], device="cuda"), inv, 4, 2, 256)
+    kc = torch.zeros(1, 2, 16, 128, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):  # table order without its sign bits
+        ops.decode_attention_rht(torch.zeros(1, 12 * 128, device="cuda"), None, 1.0, None, 12, kc, kc.clone(),
+                                 torch.tensor([0], device="cuda"), inv[:64], 8, 2, 128)
 
 
 def test_graph_capture_replays():
@@ -443,6 +457,56 @@ def test_fused_decode_with_layer_boundaries_in_the_matvec():
     assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
     for c0, c1 in zip(kc, model.k_cache):
         assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+
+
+def test_token_head_kernels():
+    """Final RMSNorm against the module's formula (model/llama.py:129-135) and the greedy pick
+    against torch.argmax: first index among equal maxima, history slot, advanced position."""
+    from qtip_amd import ops
+    from qtip_amd.llama_decode import RMSNorm
+    g = torch.Generator().manual_seed(11)
+    for n in (256, 4096, 5120, 8192):
+        x = torch.randn(1, n, generator=g).half().cuda()
+        mod = RMSNorm(n, 1e-5).cuda()
+        mod.weight.data = (1.0 + 0.1 * torch.randn(n, generator=g)).half().cuda()
+        ref = mod(x)
+        got = ops.rmsnorm(x, mod.weight, 1e-5)
+        assert got.shape == ref.shape
+        assert torch.allclose(got.float(), ref.float(), atol=0, rtol=2e-3)  # an fp16 ulp (hardware rsqrt)
+    for vocab in (512, 32000, 32003):
+        lg = torch.randn(vocab, generator=g).half().cuda()
+        top = lg.max()
+        first, second = vocab // 3, vocab // 3 + 9
+        lg[second] = top + 1
+        lg[first] = top + 1  # two equal maxima: the lower index wins
+        tok = torch.tensor([[0]], device="cuda")
+        pos = torch.tensor([40], device="cuda")
+        hist = torch.full((8,), -1, dtype=torch.int64, device="cuda")
+        ops.greedy_pick(lg, tok, pos, hist, 37)
+        assert int(tok) == first == int(torch.argmax(lg.float()))
+        assert int(pos) == 41
+        assert hist.tolist() == [-1, -1, -1, first, -1, -1, -1, -1]
+        ops.greedy_pick(lg, tok, pos, hist, 0)  # slot 41 lies outside the history: token and position only
+        assert int(pos) == 42 and hist.tolist() == [-1, -1, -1, first, -1, -1, -1, -1]
+        lg[vocab - 1] = top + 2  # the last element (the tail of an odd-sized vocabulary)
+        ops.greedy_pick(lg, tok, pos)
+        assert int(tok) == vocab - 1 and int(pos) == 43
+
+
+def test_generate_greedy_keeps_its_bookkeeping_on_the_device():
+    """Greedy decoding through the captured step (pick kernel inside the graph) returns the tokens
+    of the eager loop, and the streaming callback sees them in order."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
+    ids = torch.randint(0, cfg.vocab, (1, 7), generator=torch.Generator().manual_seed(4)).cuda()
+    seen = []
+    a, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 9, use_graph=True, callback=lambda t: seen.append(t.clone()))
+    b, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 9, use_graph=False)
+    c, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 9, use_graph=True, fused=False)
+    assert a.shape == (1, 9) and torch.equal(a, b)
+    assert len(seen) == 9 and torch.equal(torch.cat(seen, dim=1), a)
+    # the module-by-module path rounds differently; its first tokens agree on this model
+    assert torch.equal(a[:, :2], c[:, :2])
 
 
 def test_generate_sampling_and_streaming():
