@@ -16,6 +16,7 @@ Prints ONE JSON line:  value = packed bytes streamed per second (GB/s), plus
   shapes        per-matrix kernel time / GB/s / fraction of 8 TB/s
   layer         whole BitshiftLinear.forward (RHT-in + matvec + RHT-out) per matrix
   gemm_4bit     batched decompress-GEMM (batch 8/16/32) time, stream GB/s, TFLOP/s
+  decode_dense  packed -> dense fp16 weights: time, GB/s written, (read + written) / 8 TB/s
   e2e_decode    greedy decode tok/s of a random-init 7B-architecture 2-bit model
 """
 import argparse
@@ -47,8 +48,8 @@ def main():
                          "counter runs under rocprofv3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
-    ap.add_argument("--extras", default="shapes,layer,gemm,e2e",
-                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, e2e, e2e70b "
+    ap.add_argument("--extras", default="shapes,layer,gemm,decode,e2e",
+                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, e2e, e2e70b "
                          "(counter runs under rocprofv3 pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
@@ -219,6 +220,20 @@ def main():
                 del gr
             del pk4, base
         result["gemm_4bit"] = gemm
+
+    if "decode" in extras:
+        # packed -> dense fp16 weights (the reference's decode_compressed); bound by the dense write
+        dec = {}
+        for m, k in ((28672, 8192), (57344, 8192)):
+            for bits in (2, 4):
+                pkd = torch.randint(-32768, 32768, (m * k * bits // 16,), dtype=torch.int16, generator=g).to(dev)
+                ops.decode(pkd, tlut, m, k, bits)
+                gr = capture(lambda: [ops.decode(pkd, tlut, m, k, bits) for _ in range(4)])
+                us = timed(gr, 3) * 1e6 / 4
+                dec[f"{m}x{k}_k{bits}"] = {"us": round(us, 1), "written_GBps": round(m * k * 2 / us / 1e3, 1),
+                                           "frac_hbm_peak": round((m * k * 2 + m * k * bits // 8) / us / 1e3 / HBM_PEAK_GBS, 4)}
+                del gr, pkd
+        result["decode_dense"] = dec
 
     if "e2e" in extras:
         # end-to-end greedy decode, random-init Llama-2-7B architecture, every linear 2-bit

@@ -23,7 +23,26 @@ __device__ __forceinline__ float dpp_xor1(float v) {
 }
 // ---------------------------------------------------------------------------
 // decode: packed stream -> dense fp16 (m, k)
+//
+// Write-bound (2 bytes out per K/8 bytes in), so what matters is the shape of the stores.  A lane
+// decodes 4-column pieces of 16 different rows; stored as they come, a row of the matrix receives
+// 8 bytes per lane and the memory system sees partial cache lines (measured 2.4 TB/s against
+// 6.9 TB/s for a fill).  Each wave therefore turns its wave-load (32 rows x 128 columns) round
+// in LDS, a quarter (8 rows x 256 bytes) at a time: pieces go in with the 16-byte chunk index
+// xor-ed with the row (conflict free both ways), come back as one 16-byte chunk per lane, and a
+// store instruction writes four 256-byte row segments - whole cache lines only.  The 128 KiB
+// table of the matvec (32 replicas, one bank per lane) serves the lookups; the next wave-load
+// of the stream is requested before the current one is decoded.
 // ---------------------------------------------------------------------------
+constexpr size_t kDecodeLds = kLut128Bytes + kWaves * 2048;
+
+// index into W[32] (lookup order of the packed hashes) of state (R, t, j)
+template <int K>
+__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
+  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
+  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
+}
+
 template <int K>
 __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restrict__ out,
                                                              const uint8_t* __restrict__ packed,
@@ -31,37 +50,86 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
                                                              int m, int k) {
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-  build_lut(lut, tlut, threadIdx.x, kThreads);
+  build_lut128(lut, tlut, threadIdx.x, kThreads);
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int a = lane & 15, g = lane >> 4;
-  const uint32_t slot4 = (uint32_t)a << 2;
+  const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
+  uint8_t* stage = smem + kLut128Bytes + wave * 2048;  // this wave's [8 rows][256 bytes]
   const int nkb = k >> 5;
   const int nwl = (nkb + 3) >> 2;
   const long total = (long)(m >> 5) * nwl;  // wave-loads in the matrix
   const size_t rb_bytes = (size_t)nkb * 128 * K;
-  for (long w = (long)blockIdx.x * kWaves + wave; w < total; w += (long)gridDim.x * kWaves) {
-    const int rb = (int)(w / nwl), wl = (int)(w - (long)rb * nwl);
-    const int kb = 4 * wl + g;
-    if (kb >= nkb) continue;
-    const LaneData<K> ld =
-        load_lane<K>(packed + (size_t)rb * rb_bytes + (size_t)kb * 128 * K + a * 8 * K);
-    uint32_t st[2][4][4];
-    lane_states<K>(ld, st);
+  const long step = (long)gridDim.x * kWaves;
+  auto fetch = [&](long ww) {
+    const long wc = ww < total ? ww : total - 1;
+    const int rb = (int)(wc / nwl), wl = (int)(wc - (long)rb * nwl);
+    int kb = 4 * wl + g;
+    kb = kb < nkb ? kb : nkb - 1;  // blocks past the row's end (k / 32 not a multiple of 4) are decoded but not stored
+    return load_lane<K>(packed + (size_t)rb * rb_bytes + (size_t)kb * 128 * K + a * 8 * K);
+  };
+  // The stream is requested NB wave-loads ahead.  (Loads and stores share one in-order completion
+  // counter, so a wait for a requested wave-load also waits for the stores issued before the
+  // request; requesting 2, 4 or 8 wave-loads at a time to meet that wait less often measured no
+  // faster - the memory system, not the wave, holds the stores back.)
+  constexpr int NB = 1;
+  long w = (long)blockIdx.x * kWaves + wave;
+  LaneData<K> cur[NB];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int kh = t >> 1, mh = t & 1;
+  for (int b = 0; b < NB; ++b) cur[b] = fetch(w + b * step);
+  // piece (kh, jh) of this lane inside a quarter, and the chunk it reads back
+  const int r8 = a >> 1;
+  const int row_rd = lane >> 4, c_rd = lane & 15;
+  for (; w < total; w += NB * step) {
+    LaneData<K> nxt[NB];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int jh = j >> 1, rh = j & 1;
-        u32x2 v;
-        v[0] = lut_lookup(lut, st[0][t][j], slot4);
-        v[1] = lut_lookup(lut, st[1][t][j], slot4);
-        const size_t row = (size_t)rb * 32 + 16 * mh + 8 * rh + (a >> 1);
-        const size_t col = (size_t)kb * 32 + 16 * kh + 8 * jh + 4 * (a & 1);
-        *reinterpret_cast<u32x2*>(out + row * k + col) = v;
+    for (int b = 0; b < NB; ++b) nxt[b] = fetch(w + (NB + b) * step);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const long wb = w + b * step;
+      if (wb >= total) break;  // the same for every lane of the wave
+      const int rb = (int)(wb / nwl), wl = (int)(wb - (long)rb * nwl);
+      uint32_t P[16], W[32];
+      packed_states<K>(cur[b], P);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
+        W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
+        W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
       }
+      const bool store_ok = 4 * wl + (c_rd >> 2) < nkb;
+#pragma unroll
+      for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+        for (int rh = 0; rh < 2; ++rh) {
+#pragma unroll
+          for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+            for (int jh = 0; jh < 2; ++jh) {
+              const int t = 2 * kh + mh, j = 2 * jh + rh;
+              const int chunk = 4 * g + 2 * kh + jh;
+              u32x2 v = {W[w_index<K>(0, t, j)], W[w_index<K>(1, t, j)]};
+              *reinterpret_cast<u32x2*>(stage + r8 * 256 + ((chunk ^ r8) << 4) + 8 * (a & 1)) = v;
+            }
+          // the wave reads what its other lanes wrote: LDS serves a wave's requests in order
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int r = row_rd + 4 * i;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * 256 + ((c_rd ^ r) << 4));
+            const size_t row = (size_t)rb * 32 + 16 * mh + 8 * rh + r;
+            const size_t col = (size_t)wl * 128 + c_rd * 8;
+            if (store_ok) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + row * k + col));
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
     }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) cur[b] = nxt[b];
   }
 }
 
@@ -70,13 +138,6 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // ---------------------------------------------------------------------------
 constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
 constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a workgroup's k range
-
-// index into W[32] (lookup order of matvec_accumulate) of state (R, t, j)
-template <int K>
-__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
-  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
-  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
-}
 
 // 32 states of one wave-load.  All hashes, addresses and the 32 table reads are issued first, so
 // a read has the rest of the address arithmetic (a few hundred cycles) to come back from LDS;
@@ -897,9 +958,9 @@ hipError_t setup_once() {
     hipError_t e;
 #define QTIP_ALLOW(fn, bytes) \
   if ((e = allow_lds(fn, bytes)) != hipSuccess) return e;
-    QTIP_ALLOW((decode_kernel<2>), kLutBytes)
-    QTIP_ALLOW((decode_kernel<3>), kLutBytes)
-    QTIP_ALLOW((decode_kernel<4>), kLutBytes)
+    QTIP_ALLOW((decode_kernel<2>), kDecodeLds)
+    QTIP_ALLOW((decode_kernel<3>), kDecodeLds)
+    QTIP_ALLOW((decode_kernel<4>), kDecodeLds)
     QTIP_ALLOW((matvec_kernel<2, 2, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<3, 2, false>), kMatvecLds)
     QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
@@ -998,9 +1059,9 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
   auto* p = (const uint8_t*)packed;
   auto* t = (const uint32_t*)tlut;
   switch (bits) {
-    case 2: decode_kernel<2><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
-    case 3: decode_kernel<3><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
-    default: decode_kernel<4><<<grid, kThreads, kLutBytes, st>>>(o, p, t, m, k); break;
+    case 2: decode_kernel<2><<<grid, kThreads, kDecodeLds, st>>>(o, p, t, m, k); break;
+    case 3: decode_kernel<3><<<grid, kThreads, kDecodeLds, st>>>(o, p, t, m, k); break;
+    default: decode_kernel<4><<<grid, kThreads, kDecodeLds, st>>>(o, p, t, m, k); break;
   }
   return (int)hipGetLastError();
 }
