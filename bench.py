@@ -17,6 +17,7 @@ Prints ONE JSON line:  value = packed bytes streamed per second (GB/s), plus
   layer         whole BitshiftLinear.forward (RHT-in + matvec + RHT-out) per matrix
   gemm_4bit     batched decompress-GEMM (batch 8/16/32) time, stream GB/s, TFLOP/s
   decode_dense  packed -> dense fp16 weights: time, GB/s written, (read + written) / 8 TB/s
+  measured_ceilings  copy / fill / sum bandwidth of this box (library kernels) beside the nominal peak
   e2e_decode    greedy decode tok/s of a random-init 7B-architecture 2-bit model
 """
 import argparse
@@ -48,8 +49,8 @@ def main():
                          "counter runs under rocprofv3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
-    ap.add_argument("--extras", default="shapes,layer,gemm,decode,e2e",
-                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, e2e, e2e70b "
+    ap.add_argument("--extras", default="shapes,layer,gemm,decode,ceilings,e2e",
+                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, ceilings, e2e, e2e70b "
                          "(counter runs under rocprofv3 pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
@@ -220,6 +221,26 @@ def main():
                 del gr
             del pk4, base
         result["gemm_4bit"] = gemm
+
+    if "ceilings" in extras:
+        # what the memory system of this box delivers to simple kernels, next to the 8 TB/s nominal peak:
+        # a 1 GiB device-to-device copy (read + write), a fill (write only), a BLAS dot product and the library's
+        # own read probe (read only; the probe uses the matvec's persistent grid and non-temporal 16-byte loads)
+        src = torch.empty(1 << 28, dtype=torch.int32, device=dev).random_(0, 100)
+        dst = torch.empty_like(src)
+        nb = src.numel() * 4
+        fa, fb = src.view(torch.float32)[:1 << 27], src.view(torch.float32)[1 << 27:]  # two 512 MiB operands
+        cases = {"copy_read_plus_write": (lambda: dst.copy_(src), 2 * nb),
+                 "fill_write": (lambda: dst.fill_(1), nb),
+                 "blas_dot_read": (lambda: torch.dot(fa, fb), nb),
+                 "stream_read": (lambda: ops.probe_stream_read(src), nb)}
+        ceil = {}
+        for name, (fn, moved) in cases.items():
+            gr = capture(lambda: [fn() for _ in range(4)])
+            ceil[name + "_GBps"] = round(moved / (timed(gr, 3) / 4) / 1e9, 1)
+            del gr
+        result["measured_ceilings"] = ceil
+        del src, dst
 
     if "decode" in extras:
         # packed -> dense fp16 weights (the reference's decode_compressed); bound by the dense write

@@ -220,6 +220,12 @@ int qtip_rmsnorm(void* out_f16, const void* x_f16, const void* weight_f16, float
 int qtip_greedy_pick(const void* logits_f16, int vocab, void* tok_i64, void* pos_i64, void* history_i64,
                      long history_len, long history_base, void* stream);
 
+/* Measurement aid, no counterpart in the reference: reads `bytes` of device memory once with the
+ * matvec's kind of loads (persistent workgroups, one non-temporal 16-byte load per lane) and
+ * writes one folded word per wave to sink_u32 (16 * #CUs words).  Its duration is the stream-read
+ * ceiling of the box that bench.py prints beside the nominal HBM peak. */
+int qtip_probe_stream_read(void* sink_u32, const void* src, size_t bytes, void* stream);
+
 /* ---- packing tools (natural packing = one circular big-endian bitstream per tile, stored as
  * T*K/16 little-endian uint16 words; state i is the 16-bit window at bit i*K*V) ---------------- */
 

@@ -363,6 +363,18 @@ def greedy_pick(logits, tok, pos, history=None, history_base=0):
                                      stream_ptr(logits.device)), "qtip_greedy_pick")
 
 
+def probe_stream_read(src):
+    """Read the tensor once with the matvec's kind of loads (measurement aid: the launch's duration
+    is the stream-read ceiling bench.py reports).  Returns the per-wave folded words."""
+    require_cuda(src, "src")
+    cus = torch.cuda.get_device_properties(src.device).multi_processor_count
+    sink = torch.empty(16 * cus, dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        check(lib().qtip_probe_stream_read(_ptr(sink), _ptr(src), src.numel() * src.element_size(),
+                                           stream_ptr(src.device)), "qtip_probe_stream_read")
+    return sink
+
+
 # ---- packing tools ---------------------------------------------------------------------------
 
 def repack(packed, m, k, bits, to_kernel=True):
