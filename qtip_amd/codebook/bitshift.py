@@ -172,6 +172,10 @@ class bitshift_codebook(nn.Module):
 class BitshiftLinear(nn.Module):
 
     max_rows = 65535  # rows per launch of the transform / GEMM kernels (grid limit)
+    # from this many rows on the dense decode + library GEMM is faster than the fused
+    # decompress-GEMM, which runs in passes of 32 rows (measured crossover 128-192 rows for the
+    # Llama-2 7B and 70B matrices at 2 and 4 bits)
+    dense_rows_min = 160
 
     def __init__(self, td_x, td_y, L, K, V, tlut_bits, decode_mode, dtype=torch.float16, tlut=None,
                  has_kernel=False):
@@ -295,8 +299,14 @@ class BitshiftLinear(nn.Module):
                 # partial sums (if any) are added by the output transform on load
                 y = ops.decompress_matvec_parts(trellis.reshape(-1), xt.reshape(-1), tl.reshape(-1), m, n, self.cb.K)
                 in_parts = y.shape[0]
-            else:
+            elif bs < self.dense_rows_min:
                 y = ops.decompress_gemm(trellis.reshape(-1), xt, tl, m, n, self.cb.K, round_f16=True)
+            else:
+                # many rows: decode once to dense fp16 and let the BLAS library multiply, which is
+                # what the reference does for every batch (bitshift.py:476-489)
+                hatW = ops.decode(trellis.reshape(-1), tl.reshape(-1), m, n, self.cb.K)
+                y = (xt @ hatW.T).float()
+                del hatW
         else:
             if mode == 'eval':
                 hatW = self.get_hatW_natural(trellis, m, n)
@@ -364,8 +374,10 @@ class BitshiftLinearKernelAG(torch.autograd.Function):
         if x.shape[0] == 1:
             y = ops.decompress_matvec(trellis.reshape(-1), x.reshape(-1), tlut.reshape(-1), m, n, K).view(1, m)
             y = y.to(torch.float16)
-        else:
+        elif x.shape[0] < BitshiftLinear.dense_rows_min:
             y = ops.decompress_gemm(trellis.reshape(-1), x, tlut.reshape(-1), m, n, K, round_f16=True).to(torch.float16)
+        else:
+            y = x @ ops.decode(trellis.reshape(-1), tlut.reshape(-1), m, n, K).T
         return y.view(*input.shape[:-1], m)
 
     @staticmethod

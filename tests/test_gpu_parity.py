@@ -635,6 +635,34 @@ def test_forward_empty_and_slabbed_batches():
     assert (slabbed.float() - whole.float()).abs().max() <= 2e-3 * whole.float().abs().max()
 
 
+def test_forward_many_rows_decodes_and_multiplies():
+    """From BitshiftLinear.dense_rows_min rows on the layer decodes to dense fp16 and multiplies
+    with the BLAS library (the reference's route for every batch, bitshift.py:476-489): same
+    result as the fused decompress-GEMM and as the oracle's dense layer."""
+    from qtip_amd.codebook.bitshift import BitshiftLinear, BitshiftLinearKernelAG
+    from qtip_amd.utils import matmul_had as mh
+    m, k, K = 512, 1024, 2
+    L = make_layer(m, k, K, seed=9)
+    mod = BitshiftLinear(16, 16, 16, K, 2, 9, "quantlut_sym", tlut=dev(L["tlut"]), has_kernel=True)
+    hl, Kl = mh.get_hadK(k)
+    hr, Kr = mh.get_hadK(m)
+    args = (dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), hl, hr, Kl, Kr, 0, 8)
+    rows = BitshiftLinear.dense_rows_min + 9
+    x = torch.randn(rows, k, generator=torch.Generator().manual_seed(2)).half()
+    dense = mod(x.cuda(), *args)
+    mod.dense_rows_min = 10**9
+    fused = mod(x.cuda(), *args)
+    assert dense.shape == fused.shape == (rows, m)
+    assert_close(dense.float().cpu().numpy(), fused.float().cpu().numpy(), 5e-3, 5e-4)
+    ref = O.bitshift_linear_forward(x[:4].numpy(), L["packed"], L["SU"], L["SV"], L["tlut"], K)
+    assert_close(dense[:4].cpu().numpy(), ref)
+    lut = mod.cb.lut.cuda() if hasattr(mod.cb, "lut") else None
+    if lut is not None:
+        a = BitshiftLinearKernelAG.apply(x.cuda(), dev(L["packed"]), m, k, 16, 9, K, 2, lut)
+        b = BitshiftLinearKernelAG.apply(x[:8].cuda(), dev(L["packed"]), m, k, 16, 9, K, 2, lut)
+        assert_close(a[:8].float().cpu().numpy(), b.float().cpu().numpy(), 5e-3, 5e-4)
+
+
 @pytest.mark.parametrize("K", [2, 4])
 @pytest.mark.parametrize("m,k,S,Sp", [(256, 2048, None, 1), (1024, 4096, 1, 2), (4096, 4096, None, 2), (512, 8192, 4, 1),
                                       (2048, 8192, None, 3)])
