@@ -42,6 +42,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="untimed replays of the timed graph before the timed one, until this much GPU time has "
+                         "passed (the sustained clocks need tens of ms of continuous work); 0 = none")
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--workload", choices=["70b", "7b"], default="70b")
     ap.add_argument("--shape", default=None,
@@ -124,10 +127,22 @@ def main():
         return e0.elapsed_time(e1) * 1e-3 / reps
 
     # ---- headline: exactly `steps` steps in the timed region --------------
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
+    # the warm-up steps run in the same form as the timed ones (one graph) and directly before
+    # them: after the host-side pause of a graph capture the GPU needs a few milliseconds of work
+    # to be back at its running clocks, and a short timed region would measure that ramp
     graph = capture(lambda: [step(i) for i in range(args.steps)])
+    warm = capture(lambda: [step(i) for i in range(args.warmup)]) if args.warmup > 0 else None
+    torch.cuda.synchronize()
+    if warm is not None:
+        warm.replay()
+    # clock settling: the chip reaches its sustained clocks only after tens of milliseconds of
+    # continuous work (a 3 ms timed region reads 10-15 % slower than a 40 ms one), so the timed
+    # graph is replayed untimed until `settle_ms` of GPU time have passed, then timed once
+    if args.settle_ms > 0:
+        torch.cuda.synchronize()
+        one = timed(graph)
+        for _ in range(min(1000, int(args.settle_ms * 1e-3 / max(one, 1e-6)))):
+            graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     dev_s = timed(graph)
@@ -158,6 +173,7 @@ def main():
             "bytes_per_step": set_bytes,
             "weight_copies_rotated": copies,
             "timing": "one HIP graph holding all timed steps, HIP events on the launch stream",
+            "clock_settle_ms": args.settle_ms,
         },
         "roofline": {
             "bound": "hbm",

@@ -366,12 +366,17 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 // (needs 256 bytes per wave-load of the range) and read from there.
 // XFORM: 0 = x is the matvec's fp16 input, 1 = x is the layer's raw input (input transform in the
 // prologue), 2 = the previous layer's partial results (whole layer boundary in the prologue).
-template <int K, int DEPTH, bool XLDS, int XFORM = 0>
+// XHALF: the k range needs up to twice the staging area and every workgroup has exactly one unit:
+// x is staged in two halves, the second replacing the first in the middle of the unit (two more
+// barriers per launch instead of x travelling through vector loads with every wave-load, which
+// made the 28672-wide matrices 15-20 % slower).
+template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
     const uint32_t* __restrict__ tlut, int m, int k, int wl_per, int upw_q, int upw_r,
     const uint16_t* __restrict__ su = nullptr, float xscale = 1.f, const ChainArgs chain = ChainArgs{}) {
   static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
+  static_assert(!XHALF || (XLDS && !XFORM), "two-half staging is a form of the plain staged x");
   constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
@@ -456,6 +461,10 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     tw[it] = v;
   }
   u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+  u32x4 xstage2[XHALF ? 2 : 1] = {};
+  const int jh = XHALF ? (npw + 1) >> 1 : npw;  // items per wave served by the first staging
+  // wave-loads of the first staging (all of the range unless XHALF)
+  const int wlx = XHALF ? ((wl1 - wl0) < jh * kWaves ? (wl1 - wl0) : jh * kWaves) : (wl1 - wl0);
   float xraw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   ChainRegs cr;
   if constexpr (XFORM == 2) {
@@ -479,14 +488,24 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) xraw[i] *= sv[i];  // entries past k / 1024 are never read
   } else if constexpr (XLDS) {
-    // x of wave-loads [wl0, wl1): 16 bytes per thread and pass, at most 2 passes (28 KiB)
-    const int xbytes = (wl1 - wl0) * 256;
+    // x of wave-loads [wl0, wl0 + wlx): 16 bytes per thread and pass, at most 2 passes (28 KiB)
+    const int xbytes = wlx * 256;
     const int kbytes = k * 2;
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps) {
       const int o = (ps * kThreads + tid) * 16;
       if (o < xbytes && wl0 * 256 + o < kbytes)
         xstage[ps] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(x) + (size_t)wl0 * 256 + o);
+    }
+    if constexpr (XHALF) {
+      const int xbytes2 = (wl1 - wl0 - wlx) * 256;
+      const int base2 = (wl0 + wlx) * 256;
+#pragma unroll
+      for (int ps = 0; ps < 2; ++ps) {
+        const int o = (ps * kThreads + tid) * 16;
+        if (o < xbytes2 && base2 + o < kbytes)
+          xstage2[ps] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(x) + (size_t)base2 + o);
+      }
     }
   }
 #pragma unroll
@@ -518,7 +537,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     reinterpret_cast<u32x4*>(lut)[it * kThreads + tid] = v;
   }
   if constexpr (XLDS && !XFORM) {
-    const int xbytes = (wl1 - wl0) * 256;
+    const int xbytes = wlx * 256;
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps) {
       const int o = (ps * kThreads + tid) * 16;
@@ -539,6 +558,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     matvec_accumulate<K>(ld, xv, slot4, acc);
   };
   int parity = 0, c_j = 0, c_rb = rb0;
+  int c_jbase = 0;  // first item of the staging that is in LDS
   int prio_phase = wave >> 2;  // waves w, w + 4, w + 8, w + 12 share a SIMD
   for (int t = 0; t < T; t += DEPTH) {
 #pragma unroll
@@ -557,7 +577,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           if constexpr (XLDS) {
             typedef __attribute__((address_space(3))) const u32x2 lds_u32x2_t;
             u32x2 xv[4];
-            const uint32_t xa = xs_lane + (uint32_t)c_j * (kWaves * 256u);
+            const uint32_t xa = xs_lane + (uint32_t)(c_j - c_jbase) * (kWaves * 256u);
 #pragma unroll
             for (int q = 0; q < 4; ++q) xv[q] = *(lds_u32x2_t*)(uintptr_t)(xa + 16u * q);
             accumulate(buf[d], xv);
@@ -569,7 +589,22 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       // the stage's registers are refilled only after their last use, so the
       // refill reuses them in place (no copies, no wait on the new load)
       issue(d);
-      if (t + d < T && ++c_j == npw) {
+      if (t + d < T) ++c_j;
+      if constexpr (XHALF) {
+        // middle of the (only) unit: every wave has read its last x of the first half
+        if (t + d < T && c_j == jh && jh < npw) {
+          __syncthreads();
+          const int xbytes2 = (wl1 - wl0 - wlx) * 256;
+#pragma unroll
+          for (int ps = 0; ps < 2; ++ps) {
+            const int o = (ps * kThreads + tid) * 16;
+            if (o < xbytes2) *reinterpret_cast<u32x4*>(xs_lds + o) = xstage2[ps];
+          }
+          __syncthreads();
+          c_jbase = jh;
+        }
+      }
+      if (t + d < T && c_j == npw) {
         // ---- end of a unit: ragged tail, reductions, store
         // k/32 not a multiple of 4: one wave takes the partial wave-load.  Every lane takes part
         // in an MFMA, so the lanes of the missing blocks read x = 0 (the descriptor of x ends
@@ -967,6 +1002,9 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<2, 2, true, 1>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true, 1>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true, 1>), kMatvecLds + kMatvecXBytes)
@@ -996,11 +1034,13 @@ int check_common(const void* a, const void* b, const void* c, const void* d, int
   return QTIP_OK;
 }
 
-// k split S for the shape.  Cost model in units of one wave-load per wave slot (fitted to
-// measured launch times of the 7B / 70B shapes): a workgroup walks `rounds` units of nwl/S
-// wave-loads, each unit carries a fixed cost (flush, barrier, pipeline refill), a launch never
-// takes less than the latency of its first stages, and when the caller wants the summed vector
-// (not the parts) a split costs one more small launch.
+// k split S for the shape: a workgroup walks `rounds` units of nwl/S wave-loads, and when the
+// caller wants the summed vector (not the parts) a split costs one more small launch.
+// Cost model of the k split, in units of one wave-load per wave (~0.08 us), fitted to launch times
+// measured with cold weights: a unit costs its wave-loads per wave plus ~8 of fixed work (flush,
+// barrier, stores; ~2 more when the output is a partial vector), a k range longer than the x
+// staging area of LDS makes every wave-load ~20 % dearer (x then travels through vector loads),
+// and a launch does not get shorter than ~24 however little each workgroup has to do.
 int choose_split(int m, int k, int bits, int cus, bool summed) {
   (void)bits;
   const int nrb = m >> 5;
@@ -1011,9 +1051,11 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
     if (nwl / S < kWaves && S > 1) break;  // keep at least one wave-load per wave
     const long units = (long)nrb * S;
     const long rounds = (units + cus - 1) / cus;
-    const double per_unit = (double)nwl / S + 12.0 + (S > 1 ? 4.0 : 0.0);
+    const int wl_per = (nwl + S - 1) / S;
+    const bool x_in_lds = (size_t)wl_per * 256 <= kMatvecXBytes;
+    const double per_unit = (double)nwl / S * (x_in_lds ? 1.0 : 1.2) + 8.0 + (S > 1 ? 2.0 : 0.0);
     double cost = rounds * per_unit;
-    if (cost < 40.0) cost = 40.0;
+    if (cost < 24.0) cost = 24.0;
     if (S > 1 && summed) cost += 53.0;
     if (cost < best_cost * 0.97) {
       best_cost = cost;
@@ -1122,6 +1164,14 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
       case 2: matvec_kernel<2, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
       case 3: matvec_kernel<3, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
       default: matvec_kernel<4, 2, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+    }
+  } else if (uq == 1 && ur == 0 && (size_t)((((wl_per + kWaves - 1) / kWaves) + 1) >> 1) * kWaves * 256 <= kMatvecXBytes) {
+    // one unit per workgroup and a k range of at most twice the staging area: x in two halves
+    const size_t lds = kMatvecLds + kMatvecXBytes;
+    switch (bits) {
+      case 2: matvec_kernel<2, 2, true, 0, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      case 3: matvec_kernel<3, 2, true, 0, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
+      default: matvec_kernel<4, 2, true, 0, true><<<g2, kThreads, lds, st>>>(dst, p, xx, t, m, k, wl_per, uq, ur); break;
     }
   } else {
     switch (bits) {
