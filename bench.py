@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch over algorithmic bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this script, each calibrated against a 256 MiB copy (summary under profiles/)
-MEASURED_TRAFFIC_RATIO = {("70b", 2): (52582.0 + 82.0) / 52224.0}
+MEASURED_TRAFFIC_RATIO = {("70b", 2): (52583.0 + 82.0) / 52224.0}
 SHAPES_70B = [("qkv", 10240, 8192), ("o", 8192, 8192), ("up_gate", 57344, 8192), ("down", 8192, 28672)]
 SHAPES_7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("up_gate", 22016, 4096), ("down", 4096, 11008)]
 
@@ -116,8 +116,12 @@ def main():
             fn()
         return gr
 
-    def timed(gr, reps=1):
+    def timed(gr, reps=1, settle_ms=0.0):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if settle_ms > 0:  # untimed replays first, see --settle-ms
+            one = timed(gr)
+            for _ in range(min(1000, int(settle_ms * 1e-3 / max(one, 1e-6)))):
+                gr.replay()
         torch.cuda.synchronize()
         e0.record()
         for _ in range(reps):
@@ -197,12 +201,16 @@ def main():
         from qtip_amd.codebook.bitshift import BitshiftLinear
         from qtip_amd.utils import matmul_had as mh
         per, layer = {}, {}
-        reps = 24
         for name, m, k in shapes:
             nbytes = m * k * K // 8
-            gr = capture(lambda: [ops.decompress_matvec(packed[name][i % copies], xs[name], tlut, m, k, K,
+            # enough distinct copies of this one matrix to cycle through more than twice the 256 MB
+            # last-level cache, so that every launch streams from HBM
+            ncp = max(copies, -(-(600 << 20) // nbytes))
+            pks = packed[name] + [torch.roll(packed[name][0], 4099 * c) for c in range(copies, ncp)]
+            reps = ncp * max(1, 24 // ncp)
+            gr = capture(lambda: [ops.decompress_matvec(pks[i % ncp], xs[name], tlut, m, k, K,
                                                        out=outs[name]) for i in range(reps)])
-            us = timed(gr, 3) * 1e6 / reps
+            us = timed(gr, 3, args.settle_ms / 3) * 1e6 / reps
             per[name] = {"m": m, "k": k, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                          "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
             del gr
@@ -212,11 +220,11 @@ def main():
             SU = torch.sign(torch.randn(k, generator=g) + 1e-5).half().to(dev)
             SV = (torch.sign(torch.randn(m, generator=g) + 1e-5) / k**0.5).float().to(dev)
             inp = torch.randn(1, k, generator=g).half().to(dev)
-            gr = capture(lambda: [mod(inp, packed[name][i % copies].view(-1, 16 * K), SU, SV, hl, hr, Kl, Kr, 0, 8)
+            gr = capture(lambda: [mod(inp, pks[i % ncp].view(-1, 16 * K), SU, SV, hl, hr, Kl, Kr, 0, 8)
                                   for i in range(reps)])
-            lus = timed(gr, 3) * 1e6 / reps
+            lus = timed(gr, 3, args.settle_ms / 3) * 1e6 / reps
             layer[name] = {"us": round(lus, 2), "GBps": round(nbytes / lus / 1e3, 1)}
-            del gr
+            del gr, pks
         result["shapes"] = per
         result["layer"] = layer
 
@@ -230,7 +238,7 @@ def main():
             for B in (8, 16, 32):
                 X = torch.randn(B, k, generator=g).half().to(dev)
                 gr = capture(lambda: [ops.decompress_gemm(pk4[i % 6], X, tlut, m, k, 4) for i in range(12)])
-                us = timed(gr, 3) * 1e6 / 12
+                us = timed(gr, 3, args.settle_ms / 3) * 1e6 / 12
                 tf = 2.0 * m * k * B / us / 1e6
                 gemm[f"{m}x{k}_b{B}"] = {"us": round(us, 2), "stream_GBps": round(nbytes / us / 1e3, 1),
                                          "TFLOPs": round(tf, 1), "frac_mfma_f16_peak": round(tf / 2500.0, 4)}
@@ -253,7 +261,7 @@ def main():
         ceil = {}
         for name, (fn, moved) in cases.items():
             gr = capture(lambda: [fn() for _ in range(4)])
-            ceil[name + "_GBps"] = round(moved / (timed(gr, 3) / 4) / 1e9, 1)
+            ceil[name + "_GBps"] = round(moved / (timed(gr, 3, args.settle_ms / 3) / 4) / 1e9, 1)
             del gr
         result["measured_ceilings"] = ceil
         del src, dst
@@ -266,7 +274,7 @@ def main():
                 pkd = torch.randint(-32768, 32768, (m * k * bits // 16,), dtype=torch.int16, generator=g).to(dev)
                 ops.decode(pkd, tlut, m, k, bits)
                 gr = capture(lambda: [ops.decode(pkd, tlut, m, k, bits) for _ in range(4)])
-                us = timed(gr, 3) * 1e6 / 4
+                us = timed(gr, 3, args.settle_ms / 3) * 1e6 / 4
                 dec[f"{m}x{k}_k{bits}"] = {"us": round(us, 1), "written_GBps": round(m * k * 2 / us / 1e3, 1),
                                            "frac_hbm_peak": round((m * k * 2 + m * k * bits // 8) / us / 1e3 / HBM_PEAK_GBS, 4)}
                 del gr, pkd
