@@ -116,6 +116,21 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
                                        const void* su_f16, float scale_in, void* x_out_f16,
                                        void* stream);
 
+/* qtip_decompress_matvec_parts_chain for up to three matrices that share their input and
+ * differ in everything else - the separate q / k / v (or gate / up) projections of the published
+ * checkpoints (model/llama.py:246-262 q_proj, k_proj, v_proj; :389-400 gate_proj, up_proj), each a
+ * QuantizedLinear with its own trellis, table and sign vectors - in ONE launch: the workgroups
+ * are shared out among the matrices in proportion to their rows.  packed / tlut / su_f16 / m are
+ * HOST arrays of ngroups (1..3) device pointers / row counts; parts is [nparts][sum of m] fp32,
+ * matrix g's rows following those of matrix g - 1; the boundary arguments are those of
+ * qtip_decompress_matvec_parts_chain (one residual stream, one x_out). */
+int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* const* packed,
+                                       const void* const* tlut, const void* const* su_f16, const int* m,
+                                       int k, int bits, int nparts, const float* prev_parts,
+                                       int prev_nparts, size_t prev_part_stride, const float* post_f32,
+                                       float scale_out, const void* residual_f16, const void* norm_weight_f16,
+                                       float eps, float scale_in, void* x_out_f16, void* stream);
+
 /* Bytes of scratch qtip_decompress_gemm wants for this shape (0 when it does not split k). */
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch);
 

@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _lib = None
 
@@ -35,6 +35,10 @@ _SIGNATURES = {
                                            [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_float,
                                             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_float,
                                             ctypes.c_void_p, ctypes.c_void_p]),
+    "qtip_decompress_matvec_group_chain": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 4 +
+                                           [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t,
+                                            ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p,
+                                            ctypes.c_float, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p]),
     "qtip_decompress_matvec": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
                                [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "qtip_gemm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),

@@ -262,6 +262,25 @@ struct ChainArgs {
   float scale_out, eps;
   int in_parts;
 };
+// Up to three matrices with the same k and bit width in one launch (the separate q / k / v or
+// gate / up projections of a decoder layer): the workgroups blockIdx.y in
+// [wg_begin[g], wg_begin[g + 1]) serve matrix g with its own stream, table, sign vector and
+// output rows; everything else (k split, layer boundary, x_out) is shared.
+struct GroupArgs {
+  float* dst[3];              // first output row of the matrix inside a partial result
+  const uint8_t* packed[3];
+  const uint32_t* tlut[3];
+  const uint16_t* su[3];
+  int m[3];
+  int wg_begin[4];
+  int upw_q[3], upw_r[3];
+  size_t part_stride;         // floats between partial results
+};
+template <typename T>
+__device__ __forceinline__ T pick3(const T (&a)[3], int g) {
+  return g == 0 ? a[0] : (g == 1 ? a[1] : a[2]);
+}
+
 struct ChainRegs {  // a thread's operands, k / 1024 <= 8 consecutive elements each
   float v[8], pv[8], rv[8], wv[8], sv[8];
 };
@@ -370,12 +389,24 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 // x is staged in two halves, the second replacing the first in the middle of the unit (two more
 // barriers per launch instead of x travelling through vector loads with every wave-load, which
 // made the 28672-wide matrices 15-20 % slower).
-template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false>
+template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false, bool GROUP = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
-    float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
-    const uint32_t* __restrict__ tlut, int m, int k, int wl_per, int upw_q, int upw_r,
-    const uint16_t* __restrict__ su = nullptr, float xscale = 1.f, const ChainArgs chain = ChainArgs{}) {
+    float* __restrict__ dst_, const uint8_t* __restrict__ packed_, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut_, int m_, int k, int wl_per, int upw_q_, int upw_r_,
+    const uint16_t* __restrict__ su_ = nullptr, float xscale = 1.f, const ChainArgs chain = ChainArgs{},
+    const GroupArgs grp = GroupArgs{}) {
   static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
+  static_assert(!GROUP || XFORM == 2, "grouped launches exist for the layer-boundary form");
+  // the matrix this workgroup serves (uniform: scalar selects on kernel arguments)
+  int gi = 0;
+  if constexpr (GROUP) gi = (int)blockIdx.y >= grp.wg_begin[2] ? 2 : ((int)blockIdx.y >= grp.wg_begin[1] ? 1 : 0);
+  float* __restrict__ dst = GROUP ? pick3(grp.dst, gi) : dst_;
+  const uint8_t* __restrict__ packed = GROUP ? pick3(grp.packed, gi) : packed_;
+  const uint32_t* __restrict__ tlut = GROUP ? pick3(grp.tlut, gi) : tlut_;
+  const uint16_t* __restrict__ su = GROUP ? pick3(grp.su, gi) : su_;
+  const int m = GROUP ? pick3(grp.m, gi) : m_;
+  const int upw_q = GROUP ? pick3(grp.upw_q, gi) : upw_q_;
+  const int upw_r = GROUP ? pick3(grp.upw_r, gi) : upw_r_;
   static_assert(!XHALF || (XLDS && !XFORM), "two-half staging is a form of the plain staged x");
   constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
   extern __shared__ __align__(16) uint8_t smem[];
@@ -397,8 +428,10 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 
   // grid = (S, workgroups per k range): no integer division on the way to the first loads
   const int s = blockIdx.x;
-  const int rb0 = blockIdx.y;
-  const int rb_step = gridDim.y;
+  const int wg0 = GROUP ? (gi == 0 ? 0 : (gi == 1 ? grp.wg_begin[1] : grp.wg_begin[2])) : 0;
+  const int rb0 = (int)blockIdx.y - wg0;
+  const int rb_step = GROUP ? (gi == 0 ? grp.wg_begin[1] : (gi == 1 ? grp.wg_begin[2] : grp.wg_begin[3])) - wg0
+                            : (int)gridDim.y;
   const int wl0 = s * wl_per;
   const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
   const int wl1f = wl1 < nfull ? wl1 : nfull;           // end of the full wave-loads
@@ -408,7 +441,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const int w_first = wl0 + wave;
   const int nvj = w_first < wl1f ? (wl1f - w_first + kWaves - 1) / kWaves : 0;  // real items per unit
   const bool tail_wave = wl1 > nfull && ((nfull - wl0) % kWaves) == wave;
-  float* out_s = dst + (size_t)s * m;
+  float* out_s = dst + (size_t)s * (GROUP ? grp.part_stride : (size_t)m);
 
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
@@ -1002,6 +1035,9 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<2, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
@@ -1069,7 +1105,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 11; }
+int qtip_abi_version(void) { return 12; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -1242,6 +1278,115 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
   c.eps = eps;
   c.in_parts = prev_nparts;
   return launch_matvec(parts, packed, su_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale_in, &c);
+}
+
+int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* const* packed,
+                                       const void* const* tlut, const void* const* su_f16, const int* m,
+                                       int k, int bits, int nparts, const float* prev_parts,
+                                       int prev_nparts, size_t prev_part_stride, const float* post,
+                                       float scale_out, const void* residual_f16, const void* norm_w_f16,
+                                       float eps, float scale_in, void* x_out_f16, void* stream) {
+  if (!parts || !packed || !tlut || !su_f16 || !m) return QTIP_E_NULL;
+  if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
+  long m_total = 0;
+  for (int g = 0; g < ngroups; ++g) {
+    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits);
+    if (rc) return rc;
+    if (!aligned16(su_f16[g])) return QTIP_E_ALIGN;
+    m_total += m[g];
+  }
+  if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
+  if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
+  if (prev_nparts < 1 || prev_nparts > kMaxSplit || x_out_f16 == residual_f16) return QTIP_E_SHAPE;
+  if (!aligned16(prev_parts) || !aligned16(post) || !aligned16(residual_f16) || !aligned16(norm_w_f16) ||
+      !aligned16(x_out_f16) || ((prev_part_stride * sizeof(float)) & 15u))
+    return QTIP_E_ALIGN;
+  ChainArgs c;
+  c.parts = prev_parts;
+  c.post = post;
+  c.residual = (const _Float16*)residual_f16;
+  c.norm_w = (const _Float16*)norm_w_f16;
+  c.x_out = (_Float16*)x_out_f16;
+  c.part_stride = prev_part_stride;
+  c.scale_out = scale_out;
+  c.eps = eps;
+  c.in_parts = prev_nparts;
+
+  // workgroups per k range, shared out in proportion to the matrices' row blocks (at least one
+  // each, never more than a matrix has row blocks)
+  const int S = nparts;
+  const int P = device_info().cus / S;
+  if (P < ngroups) return QTIP_E_SHAPE;
+  int nrb[3] = {0, 0, 0}, wg[3] = {0, 0, 0};
+  long nrb_total = 0;
+  for (int g = 0; g < ngroups; ++g) {
+    nrb[g] = m[g] >> 5;
+    nrb_total += nrb[g];
+  }
+  int used = 0;
+  for (int g = 0; g < ngroups; ++g) {
+    long w = (long)P * nrb[g] / nrb_total;
+    if (w < 1) w = 1;
+    if (w > nrb[g]) w = nrb[g];
+    wg[g] = (int)w;
+    used += wg[g];
+  }
+  while (used > P) {  // the minimum of one per matrix can overshoot
+    int big = 0;
+    for (int g = 1; g < ngroups; ++g)
+      if (wg[g] > wg[big]) big = g;
+    --wg[big];
+    --used;
+  }
+  for (bool grown = true; used < P && grown;) {  // leftovers go where a workgroup has the most units
+    grown = false;
+    int best = -1;
+    double most = 1.0;
+    for (int g = 0; g < ngroups; ++g) {
+      const double load = (double)nrb[g] / wg[g];
+      if (wg[g] < nrb[g] && load > most) {
+        most = load;
+        best = g;
+      }
+    }
+    if (best >= 0) {
+      ++wg[best];
+      ++used;
+      grown = true;
+    }
+  }
+  GroupArgs ga;
+  int begin = 0;
+  long col = 0;
+  for (int g = 0; g < 3; ++g) {
+    const int gg = g < ngroups ? g : ngroups - 1;
+    ga.dst[g] = parts + (g < ngroups ? col : 0);
+    ga.packed[g] = (const uint8_t*)packed[gg];
+    ga.tlut[g] = (const uint32_t*)tlut[gg];
+    ga.su[g] = (const uint16_t*)su_f16[gg];
+    ga.m[g] = m[gg];
+    ga.wg_begin[g] = g < ngroups ? begin : used;
+    ga.upw_q[g] = g < ngroups ? nrb[g] / wg[g] : 0;
+    ga.upw_r[g] = g < ngroups ? nrb[g] % wg[g] : 0;
+    if (g < ngroups) {
+      begin += wg[g];
+      col += m[g];
+    }
+  }
+  ga.wg_begin[3] = used;
+  ga.part_stride = (size_t)m_total;
+  const int nwl = ((k >> 5) + 3) >> 2;
+  const int wl_per = (nwl + S - 1) / S;
+  const dim3 g2((unsigned)S, (unsigned)used);
+  const size_t lds = kMatvecLds + (size_t)k * 2;
+  hipStream_t st = (hipStream_t)stream;
+  switch (bits) {
+    case 2: matvec_kernel<2, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
+    case 3: matvec_kernel<3, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
+    default: matvec_kernel<4, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
+  }
+  return (int)hipGetLastError();
 }
 
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,

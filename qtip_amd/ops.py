@@ -173,6 +173,45 @@ def decompress_matvec_parts_chain(packed, tlut, m, k, bits, prev_parts, post, sc
     return parts, x_new
 
 
+def decompress_matvec_group_chain(packed, tlut, m, k, bits, prev_parts, post, scale_out, residual, norm_weight, eps,
+                                  su, scale_in, nparts=None):
+    """decompress_matvec_parts_chain for up to three matrices that share the boundary and the
+    input (separate q / k / v or gate / up projections) in one launch.  packed, tlut, m, su: lists,
+    one entry per matrix.  Returns (parts (S, sum(m)) fp32 - matrix g's rows after those of
+    matrix g - 1 -, x_new)."""
+    n = len(packed)
+    if not (1 <= n <= 3) or len(tlut) != n or len(m) != n or len(su) != n:
+        raise ValueError("one to three matrices, with one table, row count and sign vector each")
+    dev = packed[0].device
+    for g in range(n):
+        _check_packed(packed[g], m[g], k, bits)
+        _check_tlut(tlut[g], dev)
+        require_cuda(su[g], "su", torch.float16)
+        if su[g].numel() != k or su[g].device != dev or packed[g].device != dev:
+            raise ValueError(f"every su must hold k = {k} values on {dev}")
+    require_cuda(prev_parts, "prev_parts", torch.float32)
+    require_cuda(post, "post", torch.float32)
+    require_cuda(residual, "residual", torch.float16)
+    require_cuda(norm_weight, "norm_weight", torch.float16)
+    pp = prev_parts.reshape(prev_parts.shape[0], -1)
+    if k not in RHT_IN_MATVEC_SIZES or pp.shape[1] != k:
+        raise ValueError(f"prev_parts must hold vectors of k = {k} values, k in {RHT_IN_MATVEC_SIZES}")
+    if any(t.numel() != k for t in (post, residual, norm_weight)):
+        raise ValueError(f"post, residual and norm_weight must hold k = {k} values")
+    m_total = int(sum(m))
+    S = int(nparts) if nparts is not None else matvec_split(m_total, k, bits, dev)
+    parts = torch.empty((S, m_total), dtype=torch.float32, device=dev)
+    x_new = torch.empty((1, k), dtype=torch.float16, device=dev)
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+    with torch.cuda.device(dev):
+        check(lib().qtip_decompress_matvec_group_chain(
+            _ptr(parts), n, ptrs(packed), ptrs(tlut), ptrs(su), (ctypes.c_int * n)(*[int(v) for v in m]), k, bits, S,
+            _ptr(pp), pp.shape[0], ctypes.c_size_t(pp.stride(0)), _ptr(post), ctypes.c_float(scale_out),
+            _ptr(residual), _ptr(norm_weight), ctypes.c_float(eps), ctypes.c_float(scale_in), _ptr(x_new),
+            stream_ptr(dev)), "qtip_decompress_matvec_group_chain")
+    return parts, x_new
+
+
 def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     """(batch, m) fp32 = x[batch,k] (fp16) @ decode(packed)[m,k]^T on the matrix cores."""
     _check_packed(packed, m, k, bits)

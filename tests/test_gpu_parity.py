@@ -635,6 +635,40 @@ def test_forward_empty_and_slabbed_batches():
     assert (slabbed.float() - whole.float()).abs().max() <= 2e-3 * whole.float().abs().max()
 
 
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("ms,k,S,Sp", [((512, 512, 512), 2048, None, 1), ((4096, 4096, 4096), 4096, None, 2),
+                                       ((8192, 1024, 1024), 8192, 2, 2), ((11008 - 11008 % 32, 2752), 4096, 1, 1),
+                                       ((64,), 2048, 4, 3), ((32, 32, 9600), 4096, 2, 1)])
+def test_grouped_matvec_with_layer_boundary(K, ms, k, S, Sp):
+    """Up to three matrices behind one layer boundary in one launch (separate q / k / v or
+    gate / up projections): every matrix's partial sums and the new residual stream equal the
+    single-matrix launch bit for bit (a row block is summed by one workgroup in a fixed order,
+    whichever workgroup that is)."""
+    from qtip_amd import ops
+    if K != 2 and sum(ms) > 12288:
+        pytest.skip("large shapes once")
+    g = torch.Generator().manual_seed(K + sum(ms) + Sp)
+    layers = [make_layer(m, k, K, seed=m + k + K + i) for i, m in enumerate(ms)]
+    prev = torch.randn(Sp, 1, k, generator=g).cuda()
+    SV = (torch.sign(torch.randn(k, generator=g)) * (0.5 + torch.rand(k, generator=g))).cuda()
+    res = torch.randn(1, k, generator=g).half().cuda()
+    w = (1 + 0.1 * torch.randn(k, generator=g)).half().cuda()
+    so, si, eps = 32.0 * k**-0.5, k**-0.5 / 32.0, 1e-5
+    packed = [dev(L["packed"]).reshape(-1) for L in layers]
+    tluts = [dev(L["tlut"]).reshape(-1) for L in layers]
+    sus = [dev(L["SU"]).half() for L in layers]
+    parts, x_new = ops.decompress_matvec_group_chain(packed, tluts, list(ms), k, K, prev, SV, so, res, w, eps, sus, si,
+                                                     nparts=S)
+    assert parts.shape[1] == sum(ms)
+    off = 0
+    for i, m in enumerate(ms):
+        one, x_one = ops.decompress_matvec_parts_chain(packed[i], tluts[i], m, k, K, prev, SV, so, res, w, eps, sus[i],
+                                                       si, nparts=parts.shape[0])
+        assert torch.equal(x_one, x_new)
+        assert torch.equal(parts[:, off:off + m], one), (i, m)
+        off += m
+
+
 def test_forward_many_rows_decodes_and_multiplies():
     """From BitshiftLinear.dense_rows_min rows on the layer decodes to dense fp16 and multiplies
     with the BLAS library (the reference's route for every batch, bitshift.py:476-489): same
