@@ -291,6 +291,14 @@ def main():
                                 "ms_per_token": round(1e3 / tps, 3)}
         del model
         torch.cuda.empty_cache()
+        # the layout of the published checkpoints: seven separate projections per layer (grouped launches)
+        model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev, fused=False)
+        _, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
+        result["e2e_decode_separate_projections"] = {
+            "model": "Llama-2-7B architecture, random init, 2-bit HYB, q/k/v/o/gate/up/down separate",
+            "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1), "ms_per_token": round(1e3 / tps, 3)}
+        del model
+        torch.cuda.empty_cache()
 
     if "e2e70b" in extras:
         # the same loop on the Llama-2-70B architecture (80 layers, GQA 64/8 heads, 17 GB of 2-bit weights);

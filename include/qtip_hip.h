@@ -168,6 +168,14 @@ int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_part
              int rows, int n, int order, const uint32_t* had_bits,
              const void* pre_f16, const float* post_f32, float scale, void* stream);
 
+/* qtip_rht with one `post` vector per row (post_rows_f32 is [rows][n]): the output transforms of
+ * several QuantizedLinear layers of the same size in one launch - the separate gate / up
+ * projections of a decoder layer, whose raw matvec results lie side by side in one partial-sum
+ * buffer ([in_parts][rows][n]) and whose outputs [gate | up] feed the SiLU * up transform. */
+int qtip_rht_post_rows(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
+                       int order, const uint32_t* had_bits, const float* post_rows_f32, float scale,
+                       void* stream);
+
 /* qtip_rht with the element-wise work of the layers around a QTIP linear folded in
  * (used by the end-to-end decode loop; each mode cites what it replaces):
  *   pre_mode 0  none
@@ -222,6 +230,18 @@ int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, s
                               void* k_cache_f16, void* v_cache_f16, const void* pos_i64,
                               const float* inv_freq, int heads, int kv_heads, int head_dim, int max_len,
                               void* stream);
+
+/* qtip_decode_attention_rht for separate q / k / v projections: three raw matvec results, each
+ * with the output transform of its own QuantizedLinear (q: heads * head_dim elements, k and v:
+ * kv_heads * head_dim).  parts / post_f32 / had_bits are HOST arrays of three device pointers
+ * (had_bits[i] NULL where order[i] == 1), scale / order host arrays of three values; the three
+ * results share in_parts and part_stride (they are column ranges of one partial-sum buffer, as
+ * qtip_decompress_matvec_group_chain writes it). */
+int qtip_decode_attention_rht3(void* out_f16, const float* const* parts, int in_parts, size_t part_stride,
+                               const float* const* post_f32, const float* scale,
+                               const uint32_t* const* had_bits, const int* order, void* k_cache_f16,
+                               void* v_cache_f16, const void* pos_i64, const float* inv_freq, int heads,
+                               int kv_heads, int head_dim, int max_len, void* stream);
 
 /* Final RMSNorm of the decoder for one vector: out = weight * fp16(x * rsqrt(mean(x^2) + eps))
  * (model/llama.py:129-135), n <= 16384, one launch instead of the module's six. */

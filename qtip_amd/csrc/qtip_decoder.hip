@@ -32,13 +32,17 @@ __device__ __forceinline__ float wave_reduce_sum(float v) {
 // power-of-two part) is the D-point Walsh-Hadamard transform of
 //   u[c] = sum_{jK, b'} (-1)^(bits[jK][iK] + popcount(b & b')) v[(jK * 2^logp2) + b' * D + c],
 // n additions per slice instead of a launch of its own for the whole vector.
+// XF = 1: q, k and v are slices of one transformed vector [q | k | v] (fused projection; entry 0
+// of the arrays below describes it).  XF = 2: three vectors with a transform each (separate
+// projections): q of heads * D elements, k and v of kv_heads * D.
 struct AttnXf {
-  const float* parts;
-  const float* post;
-  const uint32_t* had_bits;
+  const float* parts[3];
+  const float* post[3];
+  const uint32_t* had_bits[3];
   size_t part_stride;
-  float scale;
-  int in_parts, order, logp2, n;
+  float scale[3];
+  int order[3], logp2[3], n[3];
+  int in_parts;
 };
 
 typedef float float4a __attribute__((ext_vector_type(4)));
@@ -46,7 +50,7 @@ typedef float float4a __attribute__((ext_vector_type(4)));
 // One workgroup per query head.  qkv: [H*D | Hkv*D | Hkv*D] fp16 of the new
 // token; k_cache / v_cache: [Hkv][max_len][D] fp16; pos_ptr: position of the
 // new token (device memory, so that a recorded graph follows the position).
-template <int D, bool XF>
+template <int D, int XF>
 __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     _Float16* __restrict__ out, const _Float16* __restrict__ qkv, _Float16* __restrict__ k_cache,
     _Float16* __restrict__ v_cache, const long* __restrict__ pos_ptr,
@@ -87,29 +91,112 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     constexpr int LOGD = D == 64 ? 6 : 7;
     constexpr int G = D / 4, R = kAttnThreads / G;  // float4 column groups, chunk rows per pass
     constexpr int QP = 4, WP = 2;                   // chunk rows and partial sums in flight per thread
+    constexpr bool SEP = XF == 2;
     const int g = tid & (G - 1), r = tid >> (LOGD - 2);
-    const int logb = X.logp2 - LOGD, bmask = (1 << logb) - 1;
-    const int nrows = X.n >> LOGD;
-    // slices: q of head h, k and v of its kv head
-    const int off[3] = {h * D, (H + kvh) * D, (H + Hkv + kvh) * D};
-    int iK[3], bb[3];
+    // slices: q of head h, k and v of its kv head - of the one vector, or each of its own
+    const int off[3] = {h * D, SEP ? kvh * D : (H + kvh) * D, SEP ? kvh * D : (H + Hkv + kvh) * D};
+    int iK[3], bb[3], lgb[3];
 #pragma unroll
     for (int s3 = 0; s3 < 3; ++s3) {
-      iK[s3] = off[s3] >> X.logp2;
-      bb[s3] = (off[s3] >> LOGD) & bmask;
+      const int lp = X.logp2[SEP ? s3 : 0];
+      lgb[s3] = lp - LOGD;
+      iK[s3] = off[s3] >> lp;
+      bb[s3] = (off[s3] >> LOGD) & ((1 << lgb[s3]) - 1);
     }
-    // the epilogue's operand, requested with everything else
+    // the epilogue's operands, requested with everything else
     const int s3 = tid >> LOGD, c = tid & (D - 1);
+    const int sx = SEP ? (s3 < 3 ? s3 : 0) : 0;  // descriptor of this thread's slice
     float postv = 1.f;
-    if (tid < 3 * D && X.post) postv = X.post[off[s3 < 3 ? s3 : 0] + c];
-    // table words: with order 1 the index is 0 and the word is masked out (any readable address does)
-    const uint32_t* hb = X.order > 1 ? X.had_bits : reinterpret_cast<const uint32_t*>(X.parts);
-    const uint32_t omask = X.order > 1 ? 1u : 0u;
+    const float* postp = sx == 0 ? X.post[0] : (sx == 1 ? X.post[1] : X.post[2]);
+    if (tid < 3 * D && postp) postv = postp[off[s3 < 3 ? s3 : 0] + c];
+    const float scalev = sx == 0 ? X.scale[0] : (sx == 1 ? X.scale[1] : X.scale[2]);
     float a[3][4];  // (plain arrays: element-wise bit operations on vector-typed values went wrong in the compiler)
 #pragma unroll
     for (int s3 = 0; s3 < 3; ++s3)
 #pragma unroll
       for (int e = 0; e < 4; ++e) a[s3][e] = 0.f;
+    if constexpr (SEP) {
+      // three vectors: the rows of all three are requested in one go, one chunk row and two
+      // partial sums per slice in flight (more would spill)
+      constexpr int Q2 = 1, W2 = 2;
+      int nrows[3], maxrows = 0;
+#pragma unroll
+      for (int s3 = 0; s3 < 3; ++s3) {
+        nrows[s3] = X.n[s3] >> LOGD;
+        maxrows = nrows[s3] > maxrows ? nrows[s3] : maxrows;
+      }
+      for (int j0 = 0; j0 < maxrows; j0 += Q2 * R) {
+        float v[3][Q2][4];
+        uint32_t hw[3][Q2];
+#pragma unroll
+        for (int s3 = 0; s3 < 3; ++s3) {
+          // table words: with order 1 the index is 0 and the word is masked out (any readable address does)
+          const uint32_t* hb = X.order[s3] > 1 ? X.had_bits[s3] : reinterpret_cast<const uint32_t*>(X.parts[s3]);
+#pragma unroll
+          for (int q = 0; q < Q2; ++q) {
+            const int j = j0 + r + q * R;
+            const int jc = j < nrows[s3] ? j : 0;
+            const unsigned bit = (unsigned)(jc >> lgb[s3]) * X.order[s3] + iK[s3];
+            hw[s3][q] = hb[bit >> 5] >> (bit & 31);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[s3][q][e] = 0.f;
+          }
+        }
+        for (int w0 = 0; w0 < X.in_parts; w0 += W2) {
+          float4a raw[3][Q2][W2];
+#pragma unroll
+          for (int u = 0; u < W2; ++u) {
+            if (w0 + u < X.in_parts) {
+#pragma unroll
+              for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+                for (int q = 0; q < Q2; ++q) {
+                  const int j = j0 + r + q * R;
+                  const int jc = j < nrows[s3] ? j : 0;
+                  raw[s3][q][u] = *reinterpret_cast<const float4a*>(
+                      X.parts[s3] + (size_t)(w0 + u) * X.part_stride + ((size_t)jc << LOGD) + 4 * g);
+                }
+            } else {
+#pragma unroll
+              for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+                for (int q = 0; q < Q2; ++q) raw[s3][q][u] = float4a{0.f, 0.f, 0.f, 0.f};
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < W2; ++u)
+#pragma unroll
+            for (int s3 = 0; s3 < 3; ++s3)
+#pragma unroll
+              for (int q = 0; q < Q2; ++q) {
+                v[s3][q][0] += raw[s3][q][u].x;
+                v[s3][q][1] += raw[s3][q][u].y;
+                v[s3][q][2] += raw[s3][q][u].z;
+                v[s3][q][3] += raw[s3][q][u].w;
+              }
+        }
+#pragma unroll
+        for (int s3 = 0; s3 < 3; ++s3) {
+          const uint32_t omask = X.order[s3] > 1 ? 1u : 0u;
+          const int bmask = (1 << lgb[s3]) - 1;
+#pragma unroll
+          for (int q = 0; q < Q2; ++q) {
+            const int j = j0 + r + q * R;
+            if (j < nrows[s3]) {
+              const uint32_t sg = (((hw[s3][q] & omask) ^ (uint32_t)__builtin_popcount(bb[s3] & j & bmask)) & 1u) << 31;
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                a[s3][e] += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[s3][q][e]) ^ sg);
+            }
+          }
+        }
+      }
+    } else {
+    const int logb = lgb[0], bmask = (1 << logb) - 1;
+    const int nrows = X.n[0] >> LOGD;
+    // table words: with order 1 the index is 0 and the word is masked out (any readable address does)
+    const uint32_t* hb = X.order[0] > 1 ? X.had_bits[0] : reinterpret_cast<const uint32_t*>(X.parts[0]);
+    const uint32_t omask = X.order[0] > 1 ? 1u : 0u;
     for (int j0 = 0; j0 < nrows; j0 += QP * R) {
       float v[QP][4];
       uint32_t hw[QP][3];
@@ -121,7 +208,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
         const int jc = j < nrows ? j : 0;
 #pragma unroll
         for (int s3 = 0; s3 < 3; ++s3) {
-          const unsigned bit = (unsigned)(jc >> logb) * X.order + iK[s3];
+          const unsigned bit = (unsigned)(jc >> logb) * X.order[0] + iK[s3];
           hw[q][s3] = hb[bit >> 5] >> (bit & 31);
         }
       }
@@ -134,7 +221,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
             for (int q = 0; q < QP; ++q) {
               const int j = j0 + r + q * R;
               const int jc = j < nrows ? j : 0;
-              raw[q][u] = *reinterpret_cast<const float4a*>(X.parts + (size_t)(w0 + u) * X.part_stride +
+              raw[q][u] = *reinterpret_cast<const float4a*>(X.parts[0] + (size_t)(w0 + u) * X.part_stride +
                                                             ((size_t)jc << LOGD) + 4 * g);
             }
           } else {
@@ -166,6 +253,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
         }
       }
     }
+    }
     // rows that share a wave, then one partial slice per wave
 #pragma unroll
     for (int o = 32; o >= G; o >>= 1)
@@ -194,7 +282,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
         const float other = q_s[s3 * kMaxHeadDim + (c ^ 64)];
         y = (c & 64) ? other - y : y + other;
       }
-      h_s[s3 * D + c] = (_Float16)(y * X.scale * postv);
+      h_s[s3 * D + c] = (_Float16)(y * scalev * postv);
     }
     __syncthreads();
   }
@@ -337,7 +425,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
 
 }  // namespace
 
-static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf, void* k_cache_f16,
+static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf, int xf_mode, void* k_cache_f16,
                             void* v_cache_f16, const void* pos_i64, const float* inv_freq, int heads,
                             int kv_heads, int head_dim, int max_len, void* stream) {
   if (!out_f16 || !k_cache_f16 || !v_cache_f16 || !pos_i64 || !inv_freq) return QTIP_E_NULL;
@@ -351,25 +439,47 @@ static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf
       (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,  \
       (const long*)pos_i64, inv_freq, heads, kv_heads, max_len, ARG)
   if (xf) {
-    if (head_dim == 64) QTIP_ATTN(64, true, *xf);
-    else if (head_dim == 128) QTIP_ATTN(128, true, *xf);
-    else return QTIP_E_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return QTIP_E_SHAPE;
+    if (xf_mode == 1) {
+      if (head_dim == 64) QTIP_ATTN(64, 1, *xf); else QTIP_ATTN(128, 1, *xf);
+    } else {
+      if (head_dim == 64) QTIP_ATTN(64, 2, *xf); else QTIP_ATTN(128, 2, *xf);
+    }
   } else {
     switch (head_dim) {
-      case 64: QTIP_ATTN(64, false, AttnXf{}); break;
-      case 128: QTIP_ATTN(128, false, AttnXf{}); break;
-      default: QTIP_ATTN(256, false, AttnXf{}); break;
+      case 64: QTIP_ATTN(64, 0, AttnXf{}); break;
+      case 128: QTIP_ATTN(128, 0, AttnXf{}); break;
+      default: QTIP_ATTN(256, 0, AttnXf{}); break;
     }
   }
 #undef QTIP_ATTN
   return (int)hipGetLastError();
 }
 
+// one transformed vector of n elements: table order and log2 of the power-of-two part
+static int fill_xf_slot(AttnXf& x, int slot, const float* parts, const float* post, const uint32_t* had_bits,
+                        float scale, int order, long n, int head_dim) {
+  if (!parts || (order > 1 && !had_bits)) return QTIP_E_NULL;
+  if (order < 1 || order > 256 || n % order) return QTIP_E_SHAPE;
+  const long p2 = n / order;
+  if ((p2 & (p2 - 1)) || p2 < head_dim || n > (1 << 20)) return QTIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(parts) & 15) return QTIP_E_ALIGN;
+  x.parts[slot] = parts;
+  x.post[slot] = post;
+  x.had_bits[slot] = had_bits;
+  x.scale[slot] = scale;
+  x.order[slot] = order;
+  x.logp2[slot] = 0;
+  while ((1L << x.logp2[slot]) < p2) ++x.logp2[slot];
+  x.n[slot] = (int)n;
+  return QTIP_OK;
+}
+
 extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
                                      void* v_cache_f16, const void* pos_i64, const float* inv_freq,
                                      int heads, int kv_heads, int head_dim, int max_len, void* stream) {
   if (!qkv_f16) return QTIP_E_NULL;
-  return launch_attention(out_f16, qkv_f16, nullptr, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads,
+  return launch_attention(out_f16, qkv_f16, nullptr, 0, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads,
                           kv_heads, head_dim, max_len, stream);
 }
 
@@ -378,27 +488,37 @@ extern "C" int qtip_decode_attention_rht(void* out_f16, const float* parts, int 
                                          int order, void* k_cache_f16, void* v_cache_f16,
                                          const void* pos_i64, const float* inv_freq, int heads,
                                          int kv_heads, int head_dim, int max_len, void* stream) {
-  if (!parts || (order > 1 && !had_bits)) return QTIP_E_NULL;
-  if (in_parts < 1 || in_parts > 16 || order < 1 || order > 256 || heads < 1 || kv_heads < 1 ||
-      head_dim < 64 || head_dim > 128)
+  if (in_parts < 1 || in_parts > 16 || heads < 1 || kv_heads < 1 || head_dim < 64 || head_dim > 128 ||
+      (part_stride & 3))
     return QTIP_E_SHAPE;
-  const long n = (long)(heads + 2 * kv_heads) * head_dim;
-  if (n % order) return QTIP_E_SHAPE;
-  const long p2 = n / order;
-  if ((p2 & (p2 - 1)) || p2 < head_dim || n > (1 << 20)) return QTIP_E_SHAPE;
-  if ((reinterpret_cast<uintptr_t>(parts) & 15) || (part_stride & 3)) return QTIP_E_SHAPE;
-  AttnXf x;
-  x.parts = parts;
-  x.post = post_f32;
-  x.had_bits = had_bits;
+  AttnXf x = {};
+  const int rc = fill_xf_slot(x, 0, parts, post_f32, had_bits, scale, order,
+                              (long)(heads + 2 * kv_heads) * head_dim, head_dim);
+  if (rc) return rc;
   x.part_stride = part_stride;
-  x.scale = scale;
   x.in_parts = in_parts;
-  x.order = order;
-  x.logp2 = 0;
-  while ((1L << x.logp2) < p2) ++x.logp2;
-  x.n = (int)n;
-  return launch_attention(out_f16, nullptr, &x, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
+  return launch_attention(out_f16, nullptr, &x, 1, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
+                          head_dim, max_len, stream);
+}
+
+extern "C" int qtip_decode_attention_rht3(void* out_f16, const float* const* parts, int in_parts,
+                                          size_t part_stride, const float* const* post_f32, const float* scale,
+                                          const uint32_t* const* had_bits, const int* order, void* k_cache_f16,
+                                          void* v_cache_f16, const void* pos_i64, const float* inv_freq,
+                                          int heads, int kv_heads, int head_dim, int max_len, void* stream) {
+  if (!parts || !post_f32 || !scale || !had_bits || !order) return QTIP_E_NULL;
+  if (in_parts < 1 || in_parts > 16 || heads < 1 || kv_heads < 1 || head_dim < 64 || head_dim > 128 ||
+      (part_stride & 3))
+    return QTIP_E_SHAPE;
+  AttnXf x = {};
+  for (int s = 0; s < 3; ++s) {
+    const long n = (long)(s == 0 ? heads : kv_heads) * head_dim;
+    const int rc = fill_xf_slot(x, s, parts[s], post_f32[s], had_bits[s], scale[s], order[s], n, head_dim);
+    if (rc) return rc;
+  }
+  x.part_stride = part_stride;
+  x.in_parts = in_parts;
+  return launch_attention(out_f16, nullptr, &x, 2, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
                           head_dim, max_len, stream);
 }
 

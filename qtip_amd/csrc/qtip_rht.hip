@@ -41,6 +41,7 @@ struct RhtParams {
   const _Float16* residual;  // or null
   size_t part_stride;
   size_t in_row_stride;      // elements between consecutive rows of `in`
+  size_t post_row_stride;    // elements between the rows' `post` vectors (0: one vector for all rows)
   float scale, eps;
   int in_parts, n, order, logA, pp, pre_mode;
   // from the host (divisions and search loops in the prologue of a latency-bound kernel are time on
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
   if (active) {
     const size_t idx = ((size_t)(iK0 + row) * A + iA) * pp + cfin;
     float o = y * P.scale;
-    if (P.post) o *= P.post[idx];
+    if (P.post) o *= P.post[r * P.post_row_stride + idx];
     TOut* op = reinterpret_cast<TOut*>(P.out) + r * (size_t)n + idx;
     if (FUSED && P.residual) {
       const float res = (float)P.residual[r * (size_t)n + idx];
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   const size_t oidx = ((size_t)iK * A + iA) * pp + cfin;
   float postv = 1.f, resv = 0.f;
   if (active) {
-    if (P.post) postv = P.post[oidx];
+    if (P.post) postv = P.post[r * P.post_row_stride + oidx];
     if (FUSED && P.residual) resv = (float)P.residual[r * (size_t)n + oidx];
   }
 
@@ -669,6 +670,26 @@ int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_part
   P.had_bits = had_bits;
   P.pre = (const _Float16*)pre_f16;
   P.post = post_f32;
+  P.part_stride = (size_t)(rows > 0 ? rows : 0) * (size_t)(n > 0 ? n : 0);
+  P.in_row_stride = (size_t)(n > 0 ? n : 0);
+  P.scale = scale;
+  P.in_parts = in_parts;
+  P.n = n;
+  P.order = order;
+  P.pre_mode = PRE_NONE;
+  return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+int qtip_rht_post_rows(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
+                       int order, const uint32_t* had_bits, const float* post_rows_f32, float scale,
+                       void* stream) {
+  if (!post_rows_f32) return QTIP_E_NULL;
+  RhtParams P{};
+  P.out = out;
+  P.in = in;
+  P.had_bits = had_bits;
+  P.post = post_rows_f32;
+  P.post_row_stride = (size_t)(n > 0 ? n : 0);
   P.part_stride = (size_t)(rows > 0 ? rows : 0) * (size_t)(n > 0 ? n : 0);
   P.in_row_stride = (size_t)(n > 0 ? n : 0);
   P.scale = scale;

@@ -150,6 +150,8 @@ class DecoderLayer(nn.Module):
         layer whose qkv matvec this one launches.  Returns (x, qkv partial sums for the next layer)."""
         cfg = self.cfg
         f = self._fused_linears()
+        if self.grouped_ok():
+            return self._decode_grouped(x, k_cache, v_cache, pos, inv_freq, qkv_parts, next_layer)
         if self.fused:
             if qkv_parts is None:
                 qkv_parts = f['qkv'].matvec(f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps))
@@ -181,6 +183,72 @@ class DecoderLayer(nn.Module):
             parts = f['down'].matvec(f['down'].transform_in(ug, ops.PRE_SILU_MUL))
             return f['down'].chain_matvec(parts, x, nq, next_layer.input_norm.weight, cfg.eps)
         return f['down'](ug, ops.PRE_SILU_MUL, residual=x), None
+
+    # ---- separate projections (the layout of the published checkpoints) in grouped launches
+
+    def grouped_ok(self):
+        """Separate q / k / v and gate / up projections that the grouped launches cover: all
+        quantized, power-of-two hidden size, equal bit widths inside a group, output transforms
+        that fit the attention prologue."""
+        if not hasattr(self, "_grouped"):
+            ok = not self.fused
+            if ok:
+                f = self._fused_linears()
+                cfg = self.cfg
+                ok = not any(l.dense for l in f.values()) and cfg.hidden in ops.RHT_IN_MATVEC_SIZES
+                if ok:
+                    q, k, v, g, u, o, d = (f[n] for n in ('q_proj', 'k_proj', 'v_proj', 'gate_proj', 'up_proj', 'o',
+                                                          'down'))
+                    ok = (q.K == k.K == v.K and g.K == u.K and g.m == u.m and g.Kr == u.Kr
+                          and all(l.Kl == 1 and l.n == cfg.hidden for l in (q, k, v, g, u))
+                          and all(l.out_transform_fits_attention(cfg.head_dim) for l in (q, k, v))
+                          and o.Kr == 1 and o.m == cfg.hidden and d.Kr == 1 and d.m == cfg.hidden
+                          and all(l.SU.dtype == torch.float16 for l in (q, k, v, g, u)))
+                    if ok:
+                        self._sv_gate_up = torch.stack([g.SV, u.SV]).contiguous()
+            self._grouped = ok
+        return self._grouped
+
+    def _group_chain(self, names, prev_parts, prev, residual, norm_weight):
+        """One launch: boundary after `prev` (its output transform, residual, RMSNorm) and the
+        matvecs of the projections `names`, which share that input."""
+        f = self._fused_linears()
+        ls = [f[n] for n in names]
+        return ops.decompress_matvec_group_chain(
+            [l.trellis for l in ls], [l.tlut for l in ls], [l.m for l in ls], ls[0].n, ls[0].K, prev_parts, prev.SV,
+            (prev.m**-0.5) * 32.0, residual, norm_weight, self.cfg.eps, [l.SU for l in ls], (ls[0].n**-0.5) / 32.0)
+
+    def _decode_grouped(self, x, k_cache, v_cache, pos, inv_freq, qkv_parts, next_layer):
+        """decode_fused for separate projections, 8 launches: [boundary + q, k, v matvecs] (by the
+        previous layer), attention with the three output transforms in its prologue, o matvec with
+        its input transform, [boundary + gate, up matvecs], both output transforms, [SiLU * up +
+        transform], down matvec.  Returns (x, partial sums of the next layer's q, k, v)."""
+        cfg = self.cfg
+        f = self._fused_linears()
+        qkv = [f[n] for n in ('q_proj', 'k_proj', 'v_proj')]
+        if qkv_parts is None:  # first layer: no boundary in front of it
+            vec = torch.cat([l(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps) for l in qkv], dim=-1)
+            attn = ops.decode_attention(vec.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
+                                        cfg.head_dim)
+        else:
+            views, off = [], 0
+            for l in qkv:
+                views.append(qkv_parts[:, off:off + l.m])
+                off += l.m
+            attn = ops.decode_attention_rht3(views, [l.SV for l in qkv], [(l.m**-0.5) * 32.0 for l in qkv],
+                                             [l.br for l in qkv], [l.Kr for l in qkv], k_cache, v_cache, pos, inv_freq,
+                                             cfg.heads, cfg.kv_heads, cfg.head_dim)
+        po = f['o'].matvec_from(attn.reshape(1, -1))
+        gu_parts, x = self._group_chain(('gate_proj', 'up_proj'), po, f['o'], x, self.post_norm.weight)
+        g = f['gate_proj']
+        ug = ops.rht_post_rows(gu_parts.view(gu_parts.shape[0], 2, g.m), self._sv_gate_up, order=g.Kr, had_bits=g.br,
+                               scale=(g.m**-0.5) * 32.0)
+        pd = f['down'].matvec(f['down'].transform_in(ug.reshape(1, -1), ops.PRE_SILU_MUL))
+        if next_layer is not None and next_layer.grouped_ok():
+            parts, x = next_layer._group_chain(('q_proj', 'k_proj', 'v_proj'), pd, f['down'], x,
+                                               next_layer.input_norm.weight)
+            return x, parts
+        return f['down'].transform_out(pd, residual=x), None
 
 
 class _FusedLinear:

@@ -318,6 +318,28 @@ def rht(x, order=1, had_bits=None, pre=None, post=None, scale=None, out_dtype=No
     return out
 
 
+def rht_post_rows(parts, post_rows, order=1, had_bits=None, scale=None, out_dtype=torch.float16):
+    """Output transforms of `rows` layers of the same size in one launch: parts (S, rows, n) fp32
+    (summed over S on load), post_rows (rows, n) fp32, one vector per row.  Returns (rows, n)."""
+    require_cuda(parts, "parts", torch.float32)
+    require_cuda(post_rows, "post_rows", torch.float32)
+    if parts.dim() != 3 or post_rows.shape != parts.shape[1:]:
+        raise ValueError("parts must be (S, rows, n) and post_rows (rows, n)")
+    S, rows, n = parts.shape
+    p = n // order
+    if n % order or p & (p - 1) or rows > 65535:
+        raise ValueError(f"{n} is not {order} times a power of two, or too many rows")
+    if order > 1:
+        require_cuda(had_bits, "had_bits", torch.int32)
+    out = torch.empty((rows, n), dtype=out_dtype, device=parts.device)
+    with torch.cuda.device(parts.device):
+        check(lib().qtip_rht_post_rows(_ptr(out), _DT[out_dtype], _ptr(parts), _DT[torch.float32], S, rows, n, order,
+                                       _ptr(had_bits), _ptr(post_rows),
+                                       ctypes.c_float(scale if scale is not None else n ** -0.5),
+                                       stream_ptr(parts.device)), "qtip_rht_post_rows")
+    return out
+
+
 def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head_dim):
     """Attention output (heads*head_dim,) fp16 of one new token: RoPE, cache write at `pos`
     (device int64 tensor with one element) and attention over cache slots 0..pos in one launch.
@@ -368,6 +390,42 @@ def decode_attention_rht(parts, post, scale, had_bits, order, k_cache, v_cache, 
                                               _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), heads,
                                               kv_heads, head_dim, max_len, stream_ptr(parts.device)),
               "qtip_decode_attention_rht")
+    return out
+
+
+def decode_attention_rht3(parts, post, scale, had_bits, order, k_cache, v_cache, pos, inv_freq, heads, kv_heads,
+                          head_dim):
+    """decode_attention_rht for separate q / k / v projections: parts, post, scale, had_bits and
+    order are 3-element lists (q, k, v); the three `parts` are (S, n_i) fp32 views into one
+    partial-sum buffer (same number of parts and the same row stride)."""
+    for i in range(3):
+        require_cuda(parts[i], "parts", torch.float32, contiguous=False)
+        if post[i] is not None:
+            require_cuda(post[i], "post", torch.float32)
+        if had_bits[i] is not None:
+            require_cuda(had_bits[i], "had_bits", torch.int32)
+        n = (heads if i == 0 else kv_heads) * head_dim
+        if parts[i].dim() != 2 or parts[i].shape[1] != n or parts[i].stride(1) != 1 \
+                or parts[i].shape[0] != parts[0].shape[0] or parts[i].stride(0) != parts[0].stride(0) \
+                or (post[i] is not None and post[i].numel() != n) or (order[i] > 1 and had_bits[i] is None):
+            raise ValueError("decode_attention_rht3: inconsistent shapes")
+    require_cuda(k_cache, "k_cache", torch.float16)
+    require_cuda(v_cache, "v_cache", torch.float16)
+    require_cuda(pos, "pos", torch.int64)
+    require_cuda(inv_freq, "inv_freq", torch.float32)
+    max_len = k_cache.shape[-2]
+    if k_cache.numel() != kv_heads * max_len * head_dim or v_cache.shape != k_cache.shape \
+            or inv_freq.numel() != head_dim // 2 or pos.numel() != 1:
+        raise ValueError("decode_attention_rht3: inconsistent shapes")
+    dev = parts[0].device
+    out = torch.empty(heads * head_dim, dtype=torch.float16, device=dev)
+    vp = lambda ts: (ctypes.c_void_p * 3)(*[t.data_ptr() if t is not None else None for t in ts])
+    with torch.cuda.device(dev):
+        check(lib().qtip_decode_attention_rht3(_ptr(out), vp(parts), parts[0].shape[0], parts[0].stride(0), vp(post),
+                                               (ctypes.c_float * 3)(*[float(v) for v in scale]), vp(had_bits),
+                                               (ctypes.c_int * 3)(*[int(v) for v in order]), _ptr(k_cache),
+                                               _ptr(v_cache), _ptr(pos), _ptr(inv_freq), heads, kv_heads, head_dim,
+                                               max_len, stream_ptr(dev)), "qtip_decode_attention_rht3")
     return out
 
 

@@ -440,6 +440,43 @@ def test_decode_attention_with_output_transform_in_prologue(heads, kv_heads, D, 
     assert_close(got.float().cpu().numpy(), ref.float().cpu().numpy(), 5e-3, 1e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,D,S", [(32, 32, 128, 1), (64, 8, 128, 2), (24, 24, 128, 3), (16, 4, 64, 1),
+                                                 (40, 40, 128, 2)])
+def test_decode_attention_with_three_output_transforms_in_prologue(heads, kv_heads, D, S):
+    """Separate q / k / v projections: attention on the three raw partial-sum vectors (column
+    ranges of one buffer) == the three output transforms as launches of their own, then attention."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits
+    ns = [heads * D, kv_heads * D, kv_heads * D]
+    max_len, pos = 128, 33
+    g = torch.Generator().manual_seed(sum(ns) + S)
+    buf = (torch.randn(S, sum(ns), generator=g) * 0.3).cuda()
+    offs = [0, ns[0], ns[0] + ns[1]]
+    parts = [buf[:, o:o + n] for o, n in zip(offs, ns)]
+    posts = [(torch.sign(torch.randn(n, generator=g) + 1e-5) * (1.0 + 0.1 * torch.rand(n, generator=g))).cuda()
+             for n in ns]
+    orders, bits, scales, vecs = [], [], [], []
+    for p, post, n in zip(parts, posts, ns):
+        hadK, order = get_hadK(n)
+        b = had_bits(hadK, order, False, "cuda") if order > 1 else None
+        orders.append(order)
+        bits.append(b)
+        scales.append(n**-0.5)
+        pc = p.contiguous()
+        vecs.append(ops.rht(pc if S > 1 else pc.reshape(1, n), order=order, had_bits=b, post=post, scale=n**-0.5,
+                            out_dtype=torch.float16, in_parts=S).reshape(-1))
+    kc = (torch.randn(1, kv_heads, max_len, D, generator=g) * 0.5).half().cuda()
+    vc = torch.randn(1, kv_heads, max_len, D, generator=g).half().cuda()
+    kc1, vc1 = kc.clone(), vc.clone()
+    inv_freq = (1.0 / (10000.0**(torch.arange(0, D, 2).float() / D))).cuda()
+    p = torch.tensor([pos], device="cuda")
+    ref = ops.decode_attention(torch.cat(vecs), kc, vc, p, inv_freq, heads, kv_heads, D)
+    got = ops.decode_attention_rht3(parts, posts, scales, bits, orders, kc1, vc1, p, inv_freq, heads, kv_heads, D)
+    assert torch.allclose(kc1.float(), kc.float(), atol=2e-3, rtol=2e-3)
+    assert torch.allclose(vc1.float(), vc.float(), atol=2e-3, rtol=2e-3)
+    assert_close(got.float().cpu().numpy(), ref.float().cpu().numpy(), 5e-3, 1e-3)
+
+
 def test_fused_decode_with_layer_boundaries_in_the_matvec():
     """Hidden size 2048: the o -> up/gate and down -> next qkv boundaries run inside the following
     matvec launch (8 launches per layer); same logits and caches as the module-by-module forward."""
@@ -500,6 +537,31 @@ def test_token_head_kernels():
         lg[vocab - 1] = top + 2  # the last element (the tail of an odd-sized vocabulary)
         ops.greedy_pick(lg, tok, pos)
         assert int(tok) == vocab - 1 and int(pos) == 43
+
+
+@pytest.mark.parametrize("heads,kv_heads", [(16, 16), (16, 4)])
+def test_decode_of_separate_projections_in_grouped_launches(heads, kv_heads):
+    """The layout of the published checkpoints (seven projections per layer): the decode step on
+    grouped launches (8 per layer) gives the logits and caches of the module-by-module forward."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=2048, heads=heads, kv_heads=kv_heads, layers=3, ffn=172 * 16, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64, fused=False)
+    assert all(layer.grouped_ok() for layer in model.layers)
+    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(5, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([5], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        vc = [c.clone() for c in model.v_cache]
+        b = model.decode_fused(tok, pos)
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    for c0, c1 in zip(kc + vc, list(model.k_cache) + list(model.v_cache)):
+        assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+    out, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64, fused=False), ids, 6, use_graph=True)
+    ref, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64, fused=False), ids, 6, use_graph=False)
+    assert torch.equal(out, ref)
 
 
 def test_generate_greedy_keeps_its_bookkeeping_on_the_device():
