@@ -325,16 +325,14 @@ class _FusedLinear:
 
     def chain_matvec(self, parts, residual, nxt, norm_weight, eps):
         """(x_new, partial sums of nxt's matvec) from this layer's partial sums: the layer boundary
-        runs inside nxt's matvec launch where that is faster than a launch of its own (measured:
-        always for 4096-long vectors; for 8192 only in front of the smaller matrices, since every
-        workgroup of the matvec repeats the boundary), else chain + matvec."""
-        if nxt.n <= 4096 or nxt.m <= 16384:
-            p, x_new = ops.decompress_matvec_parts_chain(nxt.trellis, nxt.tlut, nxt.m, nxt.n, nxt.K, parts, self.SV,
-                                                         (self.m**-0.5) * 32.0, residual, norm_weight, eps, nxt.SU,
-                                                         (nxt.n**-0.5) / 32.0)
-            return x_new, p.unsqueeze(1)
-        x_new, xt = self.chain(parts, residual, nxt, norm_weight, eps)
-        return x_new, nxt.matvec(xt)
+        runs inside nxt's matvec launch.  (Timed alone, the boundary as a launch of its own followed
+        by the plain matvec is ~2 us faster in front of the largest 8192-wide matrices, since every
+        workgroup repeats the boundary; inside the decode loop the saved launch wins there too:
+        109.7 against 107.8 tok/s on the 70B architecture.)"""
+        p, x_new = ops.decompress_matvec_parts_chain(nxt.trellis, nxt.tlut, nxt.m, nxt.n, nxt.K, parts, self.SV,
+                                                     (self.m**-0.5) * 32.0, residual, norm_weight, eps, nxt.SU,
+                                                     (nxt.n**-0.5) / 32.0)
+        return x_new, p.unsqueeze(1)
 
     def __call__(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0, residual=None):
         if self.dense:
