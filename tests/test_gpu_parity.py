@@ -278,6 +278,13 @@ def test_errors_raise_not_exit():
     with pytest.raises(QtipLibraryError):  # head size 256 has no transform prologue (refused by the library)
         ops.decode_attention_rht(torch.zeros(1, 8 * 256, device="cuda"), None, 1.0, None, 1, kc, kc.clone(),
                                  torch.tensor([0], device="cuda"), inv, 4, 2, 256)
+    with pytest.raises(ValueError):  # a grouped launch takes one to three matrices
+        ops.decompress_matvec_group_chain([], [], [], 2048, 2, torch.zeros(1, 2048, device="cuda"),
+                                          torch.ones(2048, device="cuda"), 1.0,
+                                          torch.zeros(1, 2048, dtype=torch.float16, device="cuda"),
+                                          torch.ones(2048, dtype=torch.float16, device="cuda"), 1e-5, [], 1.0)
+    with pytest.raises(ValueError):  # one `post` vector per row
+        ops.rht_post_rows(torch.zeros(1, 2, 256, device="cuda"), torch.ones(256, device="cuda"))
     kc = torch.zeros(1, 2, 16, 128, dtype=torch.float16, device="cuda")
     with pytest.raises(ValueError):  # table order without its sign bits
         ops.decode_attention_rht(torch.zeros(1, 12 * 128, device="cuda"), None, 1.0, None, 12, kc, kc.clone(),
@@ -494,6 +501,24 @@ def test_fused_decode_with_layer_boundaries_in_the_matvec():
     assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
     for c0, c1 in zip(kc, model.k_cache):
         assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+
+
+def test_output_transforms_of_several_layers_in_one_launch():
+    """rht_post_rows == one qtip_rht per row with that row's post vector, bit for bit."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits
+    for n, rows, S in ((11008, 2, 1), (4096, 3, 2), (28672, 2, 2), (1024, 5, 1)):
+        g = torch.Generator().manual_seed(n + rows)
+        parts = torch.randn(S, rows, n, generator=g).cuda()
+        post = (torch.sign(torch.randn(rows, n, generator=g) + 1e-5) * (0.5 + torch.rand(rows, n, generator=g))).cuda()
+        hadK, order = get_hadK(n)
+        bits = had_bits(hadK, order, False, "cuda") if order > 1 else None
+        got = ops.rht_post_rows(parts, post, order=order, had_bits=bits, scale=n**-0.5 * 32)
+        for r in range(rows):
+            one = ops.rht(parts[:, r].contiguous() if S > 1 else parts[0, r:r + 1].contiguous(), order=order,
+                          had_bits=bits, post=post[r].contiguous(), scale=n**-0.5 * 32, out_dtype=torch.float16,
+                          in_parts=S)
+            assert torch.equal(got[r], one.reshape(-1)), (n, r)
 
 
 def test_stream_read_probe_reads_every_word_once():
