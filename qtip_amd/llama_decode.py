@@ -393,6 +393,17 @@ class LlamaDecoder(nn.Module):
         x = self.norm(x)
         return (x @ self.lm_head.T).float()
 
+    def supports_fused_decode(self):
+        """False when a layer needs what the fused decode step does not cover (per-shard
+        transforms, rcp != 0, or a layer that is not kernel-packed): generate() then decodes
+        module by module."""
+        try:
+            for layer in self.layers:
+                layer._fused_linears()
+        except NotImplementedError:
+            return False
+        return True
+
     def decode_fused(self, tok, pos, float_logits=True):
         """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab), fused kernels;
         fp32 as the reference returns them, or the fp16 values the lm_head product yields
@@ -437,6 +448,7 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
     dev = prompt_ids.device
     n = prompt_ids.shape[1]
     sampling = temperature is not None
+    fused = fused and model.supports_fused_decode()
 
     def pick(lg):
         if sampling:

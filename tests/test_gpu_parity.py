@@ -589,6 +589,21 @@ def test_decode_of_separate_projections_in_grouped_launches(heads, kv_heads):
     assert torch.equal(out, ref)
 
 
+def test_generate_falls_back_for_per_shard_transforms():
+    """A model quantised with per-shard transforms (rcp != 0) is outside the fused decode step:
+    generate() decodes it module by module instead of failing."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64)
+    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(2)).cuda()
+    assert LlamaDecoder(cfg, max_cache_len=64).supports_fused_decode()
+    model.layers[1].down.rcp.fill_(1)
+    model.layers[1].down.tp_rank.fill_(1)  # one shard: the same transform, through the general path
+    assert not model.supports_fused_decode()
+    out, _, _ = generate(model, ids, 5, use_graph=True, fused=True)
+    assert out.shape == (1, 5)
+
+
 def test_generate_greedy_keeps_its_bookkeeping_on_the_device():
     """Greedy decoding through the captured step (pick kernel inside the graph) returns the tokens
     of the eager loop, and the streaming callback sees them in order."""
