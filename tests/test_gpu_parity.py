@@ -70,7 +70,8 @@ def test_zero_stream_known_answer(K):
 
 
 @pytest.mark.parametrize("K", [2, 3, 4])
-@pytest.mark.parametrize("shape", SMALL + [(4096, 4096), (4096, 11008), (128, 28672)])
+@pytest.mark.parametrize("shape", SMALL + [(4096, 4096), (4096, 11008), (128, 28672), (64, 20480), (32, 14368),
+                                           (96, 28672 - 32)])
 @pytest.mark.parametrize("split", [True, False])
 def test_matvec_vs_oracle(K, shape, split):
     from qtip_amd import ops
