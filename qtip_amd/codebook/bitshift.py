@@ -15,7 +15,8 @@ from torch import nn
 
 from .. import ops
 from ..utils.kernel_check import has_kernel as _has_kernel
-from ..utils.matmul_had import had_bits, matmul_hadU_cuda, matmul_hadUt_cuda
+from ..utils.matmul_had import (MANY_ROWS_MIN, MANY_ROWS_MIN_ORDER, had_bits, matmul_hadU_cuda, matmul_hadUt_cuda,
+                                rht_many_rows)
 
 
 def quantlut_sym(tlut, L, nbits):
@@ -273,6 +274,9 @@ class BitshiftLinear(nn.Module):
                      and n in ops.RHT_IN_MATVEC_SIZES)
         if in_matvec:
             xt = None
+        elif fused_in and bs >= MANY_ROWS_MIN and K_left >= MANY_ROWS_MIN_ORDER:
+            xt = rht_many_rows(x, had_left, K_left, True, pre=SU, scale=(n**-0.5) / self.scale,
+                               out_dtype=torch.float16)
         elif fused_in:
             xt = ops.rht(x.contiguous(), order=K_left,
                          had_bits=had_bits(had_left, K_left, True, dev) if K_left > 1 else None,
@@ -317,7 +321,10 @@ class BitshiftLinear(nn.Module):
         # ---- output transform: (H_R y / sqrt(m)) * SV * 32, cast
         fused_out = (rcp != 2 and SV.dtype == torch.float32 and SV.device == dev
                      and input.dtype in (torch.float16, torch.float32))
-        if fused_out:
+        if fused_out and bs >= MANY_ROWS_MIN and K_right >= MANY_ROWS_MIN_ORDER and in_parts == 1:
+            out = rht_many_rows(y.reshape(bs, m), had_right, K_right, False, post=SV,
+                                scale=(m**-0.5) * self.scale, out_dtype=input.dtype)
+        elif fused_out:
             out = ops.rht(y if in_parts > 1 else y.reshape(bs, m), order=K_right,
                           had_bits=had_bits(had_right, K_right, False, dev) if K_right > 1 else None,
                           post=SV.contiguous(), scale=(m**-0.5) * self.scale, out_dtype=input.dtype,

@@ -83,6 +83,56 @@ def had_bits(hadK, K, transpose, device):
     return _bit_cache[key]
 
 
+_dense_cache = {}
+
+
+def _dense_sylvester(p, device):
+    """H_p (Sylvester order, +-1 fp32) on the device, cached."""
+    key = ("sylvester", p, torch.device(device))
+    if key not in _dense_cache:
+        h = torch.ones(1, 1)
+        while h.shape[0] < p:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        _dense_cache[key] = h.to(device)
+    return _dense_cache[key]
+
+
+# a transform with a large table order over many rows runs as library GEMMs (below); these are the
+# sizes from which that is faster than the transform kernel, whose order * A workgroups per row
+# each read the whole row.  Measured, kernel vs GEMMs: 11008 (172 x 64) 128 rows 208 vs 103 us,
+# 512 rows 809 vs 90, 2048 rows 3114 vs 280; 22016 (172 x 128) 128 rows 336 vs 102; with the small
+# orders (28 x 1024, 12 x 1024, 20 x 512) the kernel stays ahead at every row count.
+MANY_ROWS_MIN = 96
+MANY_ROWS_MIN_ORDER = 100
+_MANY_ROWS_DENSE_P = 256
+
+
+def rht_many_rows(x, hadK, K, transpose, pre=None, post=None, scale=None, out_dtype=None):
+    """post * scale * (H_K (x) H_p)(pre * x) over the last axis of a (rows, n) fp16 / fp32 tensor,
+    evaluated the way the reference does for every input (lib/utils/matmul_had.py:105-115: a
+    dense K x K matmul with the table and a Walsh-Hadamard transform of the power-of-two part) -
+    fp32 library GEMMs instead of the transform kernel.  For many rows and a large table order:
+    the kernel's per-row cost grows with the order, a GEMM's does not."""
+    rows, n = x.shape
+    p = n // K
+    dev = x.device
+    table = (hadK if hadK is not None else get_hadK(n)[0]).to(device=dev, dtype=torch.float32)
+    M = table.T if transpose else table
+    z = x.to(torch.float32)
+    if pre is not None:
+        z = z * pre.to(torch.float32)
+    z = torch.matmul(M, z.view(rows, K, p))  # the table over the K axis, batched over the rows
+    if p <= _MANY_ROWS_DENSE_P:
+        z = torch.matmul(z.reshape(rows * K, p), _dense_sylvester(p, dev))
+    else:  # long power-of-two parts: one workgroup of the transform kernel per p-point vector
+        z = z.reshape(rows * K, p).contiguous()
+        z = torch.cat([ops.rht(z[i:i + 65535], scale=1.0) for i in range(0, rows * K, 65535)], 0)
+    z = z.view(rows, n) * (n**-0.5 if scale is None else scale)
+    if post is not None:
+        z = z * post.to(torch.float32)
+    return z.to(out_dtype or x.dtype)
+
+
 torch.library.define("hadamard::hadamard", "(Tensor x, float scale) -> Tensor")
 
 
@@ -122,6 +172,9 @@ def _hadU(X, hadK, K, transpose):
     if K == 1:
         return torch.ops.hadamard.hadamard(X.contiguous(), n**(-0.5))
     x = X if X.dtype in (torch.float16, torch.float32) else X.float()
+    rows = x.numel() // n
+    if rows >= MANY_ROWS_MIN and K >= MANY_ROWS_MIN_ORDER:
+        return rht_many_rows(x.reshape(rows, n), hadK, K, transpose).to(X.dtype).reshape(X.shape)
     out = ops.rht(x.contiguous(), order=K, had_bits=had_bits(hadK, K, transpose, X.device), out_dtype=x.dtype)
     return out.to(X.dtype).reshape(X.shape)
 

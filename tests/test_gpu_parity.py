@@ -504,6 +504,24 @@ def test_fused_decode_with_layer_boundaries_in_the_matvec():
         assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
 
 
+@pytest.mark.parametrize("n,rows", [(11008, 40), (22016, 33), (28672, 32), (14336, 64), (57344, 32)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_transform_of_many_rows_through_gemms(n, rows, transpose):
+    """Large table order, many rows: the transform as library GEMMs (the reference's own
+    formulation) against the transform kernel, fp32, <= 1e-5 of the largest value."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits, rht_many_rows
+    g = torch.Generator().manual_seed(n + rows)
+    x = torch.randn(rows, n, generator=g).cuda()
+    pre = torch.sign(torch.randn(n, generator=g) + 1e-5).half().cuda()
+    post = (torch.sign(torch.randn(n, generator=g) + 1e-5) * (0.5 + torch.rand(n, generator=g))).cuda()
+    hadK, K = get_hadK(n)
+    ref = ops.rht(x, order=K, had_bits=had_bits(hadK, K, transpose, "cuda"), pre=pre, post=post, scale=n**-0.5 * 2)
+    got = rht_many_rows(x, hadK.cuda(), K, transpose, pre=pre, post=post, scale=n**-0.5 * 2)
+    assert got.shape == ref.shape and got.dtype == ref.dtype
+    assert float((got - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
 def test_output_transforms_of_several_layers_in_one_launch():
     """rht_post_rows == one qtip_rht per row with that row's post vector, bit for bit."""
     from qtip_amd import ops
