@@ -489,6 +489,81 @@ int launch_rht_l(const RhtParams& P, dim3 grid, long loads, int ri, hipStream_t 
   return (int)hipGetLastError();
 }
 
+// Many rows of a power-of-two size (n = 1024 * EPT, order 1): one workgroup per row does the
+// whole transform - register butterflies, six lane levels, one exchange through LDS that swaps
+// the wave bits with the low four lane bits, four more lane levels - and reads and writes the
+// row once.  (The forms above split a row over order * A workgroups that each read all of it:
+// right for one vector, whose transform is latency-bound, 40 times slower for a 1024-token prompt.)
+template <int EPT, typename TIn, typename TOut>
+__global__ __launch_bounds__(kRhtThreads) void rht_rows_kernel(const RhtParams P) {
+  constexpr int N = kRhtThreads * EPT;
+  __shared__ __align__(16) float xbuf[N + N / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const size_t r = blockIdx.x;
+  const int e_nat = tid * EPT;
+  const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
+  const TIn* src = reinterpret_cast<const TIn*>(P.in) + r * P.in_row_stride;
+  float v[EPT], pv[EPT];
+  auto load = [&](const TIn* p, float t[EPT]) {
+    if constexpr (sizeof(TIn) == 2) ld_f16<EPT>(reinterpret_cast<const _Float16*>(p), t);
+    else ld_f32<EPT>(reinterpret_cast<const float*>(p), t);
+  };
+  load(src + e_nat, v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) pv[i] = 1.f;
+  if (P.post) ld_f32<EPT>(P.post + r * P.post_row_stride + e_swp, pv);
+  if (P.pre) {
+    float sv[EPT];
+    ld_f16<EPT>(P.pre + e_nat, sv);
+    for (int w = 1; w < P.in_parts; ++w) {
+      float t[EPT];
+      load(src + w * P.part_stride + e_nat, t);
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) v[i] += t[i];
+    }
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) v[i] *= sv[i];
+  } else {
+    for (int w = 1; w < P.in_parts; ++w) {
+      float t[EPT];
+      load(src + w * P.part_stride + e_nat, t);
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) v[i] += t[i];
+    }
+  }
+  wht_regs<EPT>(v);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_nat + i)] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(xbuf[xidx<EPT>(e_swp + i)], 4, lane) * P.scale * pv[i];
+  TOut* dst = reinterpret_cast<TOut*>(P.out) + r * (size_t)N + e_swp;
+  if constexpr (sizeof(TOut) == 2) {
+    _Float16 h[EPT];
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) h[i] = (_Float16)v[i];
+    st_f16<EPT>(reinterpret_cast<_Float16*>(dst), h);
+  } else {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) reinterpret_cast<float*>(dst)[i] = v[i];
+  }
+}
+
+template <typename TIn, typename TOut>
+int launch_rht_rows(const RhtParams& P, int rows, hipStream_t st) {
+  switch (P.n) {
+    case 2048: rht_rows_kernel<2, TIn, TOut><<<rows, kRhtThreads, 0, st>>>(P); break;
+    case 4096: rht_rows_kernel<4, TIn, TOut><<<rows, kRhtThreads, 0, st>>>(P); break;
+    default: rht_rows_kernel<8, TIn, TOut><<<rows, kRhtThreads, 0, st>>>(P); break;
+  }
+  return (int)hipGetLastError();
+}
+
+// rows from which the one-workgroup-per-row form is used for the power-of-two sizes it covers
+constexpr int kRowsFormMin = 8;
+
 int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream) {
   if (!P.out || !P.in) return QTIP_E_NULL;
   const int n = P.n, order = P.order;
@@ -517,6 +592,20 @@ int launch_rht(RhtParams P, int out_dtype, int in_dtype, int rows, void* stream)
   P.pp = pp;
   hipStream_t st = (hipStream_t)stream;
   const bool fused = P.pre_mode != PRE_NONE || P.residual != nullptr;
+  {
+    const size_t ez = in_dtype == QTIP_F16 ? 2 : 4;
+    const bool rows_form = !fused && order == 1 && rows >= kRowsFormMin && (n == 2048 || n == 4096 || n == 8192) &&
+                           (reinterpret_cast<uintptr_t>(P.in) & 15u) == 0 && (reinterpret_cast<uintptr_t>(P.out) & 15u) == 0 &&
+                           ((P.in_row_stride * ez) & 15u) == 0 && ((P.part_stride * ez) & 15u) == 0 &&
+                           (!P.pre || (reinterpret_cast<uintptr_t>(P.pre) & 15u) == 0) &&
+                           (!P.post || ((reinterpret_cast<uintptr_t>(P.post) & 15u) == 0 && (P.post_row_stride & 3u) == 0));
+    if (rows_form) {
+      if (in_dtype == QTIP_F16 && out_dtype == QTIP_F16) return launch_rht_rows<_Float16, _Float16>(P, rows, st);
+      if (in_dtype == QTIP_F16) return launch_rht_rows<_Float16, float>(P, rows, st);
+      if (out_dtype == QTIP_F16) return launch_rht_rows<float, _Float16>(P, rows, st);
+      return launch_rht_rows<float, float>(P, rows, st);
+    }
+  }
   if (fused && out_dtype != QTIP_F16) return QTIP_E_DTYPE;  // fused forms exist for the combinations the decode loop uses
   // vectorised form: 8 columns per thread, 16-byte loads
   const size_t esz = in_dtype == QTIP_F16 ? 2 : 4;

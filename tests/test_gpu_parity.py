@@ -522,6 +522,32 @@ def test_transform_of_many_rows_through_gemms(n, rows, transpose):
     assert float((got - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("n", [2048, 4096, 8192])
+@pytest.mark.parametrize("rows,S", [(8, 1), (33, 1), (9, 3), (300, 1)])
+@pytest.mark.parametrize("dt_in,dt_out", [(torch.float16, torch.float16), (torch.float32, torch.float16),
+                                          (torch.float32, torch.float32), (torch.float16, torch.float32)])
+def test_transform_of_many_power_of_two_rows(n, rows, S, dt_in, dt_out):
+    """From 8 rows on a power-of-two transform runs one workgroup per row; against the fp64
+    Sylvester matrix (what the oracle's transform is pinned to) and the single-row forms."""
+    from qtip_amd import ops
+    import scipy.linalg
+    if S > 1 and dt_in != torch.float32:
+        pytest.skip("partial sums are fp32")
+    g = torch.Generator().manual_seed(n + rows + S)
+    x = torch.randn(S, rows, n, generator=g).to(dt_in).cuda() if S > 1 else torch.randn(rows, n, generator=g).to(dt_in).cuda()
+    pre = torch.sign(torch.randn(n, generator=g) + 1e-5).half().cuda()
+    post = (torch.sign(torch.randn(n, generator=g) + 1e-5) * (0.5 + torch.rand(n, generator=g))).cuda()
+    got = ops.rht(x, pre=pre, post=post, scale=n**-0.5, out_dtype=dt_out, in_parts=S)
+    assert got.shape == (rows, n) and got.dtype == dt_out
+    xs = x.double().sum(0) if S > 1 else x.double()
+    H = torch.from_numpy(scipy.linalg.hadamard(n).astype(np.float64)).cuda()
+    ref = ((xs * pre.double()) @ H) * n**-0.5 * post.double()
+    tol = 2e-3 if dt_out == torch.float16 else 1e-5
+    assert float((got.double() - ref).abs().max()) <= tol * float(ref.abs().max())
+    one = ops.rht(x[:, :1].contiguous() if S > 1 else x[:1], pre=pre, post=post, scale=n**-0.5, out_dtype=dt_out, in_parts=S)
+    assert float((got[:1].double() - one.double()).abs().max()) <= tol * float(ref.abs().max())
+
+
 def test_output_transforms_of_several_layers_in_one_launch():
     """rht_post_rows == one qtip_rht per row with that row's post vector, bit for bit."""
     from qtip_amd import ops
