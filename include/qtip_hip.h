@@ -131,6 +131,14 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
                                        float scale_out, const void* residual_f16, const void* norm_weight_f16,
                                        float eps, float scale_in, void* x_out_f16, void* stream);
 
+/* The plain form of the grouped launch: matrix g multiplies its own fp16 input x_f16[g] (the
+ * separate projections of a layer whose hidden size is not a power of two, where the input
+ * transforms are launches of their own).  Same layout of `parts`; every k range of x must fit the
+ * kernel's LDS staging area (k / nparts <= 14336). */
+int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* packed,
+                                 const void* const* x_f16, const void* const* tlut, const int* m, int k,
+                                 int bits, int nparts, void* stream);
+
 /* Bytes of scratch qtip_decompress_gemm wants for this shape (0 when it does not split k). */
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch);
 
@@ -175,6 +183,14 @@ int qtip_rht(void* out, int out_dtype, const void* in, int in_dtype, int in_part
 int qtip_rht_post_rows(void* out, int out_dtype, const void* in, int in_dtype, int in_parts, int rows, int n,
                        int order, const uint32_t* had_bits, const float* post_rows_f32, float scale,
                        void* stream);
+
+/* The input transforms of several QuantizedLinear layers that read the same vector, in one launch:
+ * row r of out = fp16(scale * (H_order^T (x) H_p)(pre_rows[r] * rmsnorm(in))) with the RMSNorm of
+ * qtip_rht_fused (model/llama.py:129-135) - q / k / v (or gate / up) of a decoder layer, each with
+ * its own sign vector SU (lib/codebook/bitshift.py:428-441).  in fp16[n], pre_rows fp16[rows][n]. */
+int qtip_rht_fused_pre_rows(void* out_f16, const void* in_f16, int rows, int n, int order,
+                            const uint32_t* had_bits, const void* pre_rows_f16, float scale,
+                            const void* norm_weight_f16, float eps, void* stream);
 
 /* qtip_rht with the element-wise work of the layers around a QTIP linear folded in
  * (used by the end-to-end decode loop; each mode cites what it replaces):

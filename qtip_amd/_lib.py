@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lib = None
 
@@ -39,6 +39,8 @@ _SIGNATURES = {
                                            [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t,
                                             ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p,
                                             ctypes.c_float, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p]),
+    "qtip_decompress_matvec_group": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 4 +
+                                     [ctypes.c_int] * 3 + [ctypes.c_void_p]),
     "qtip_decompress_matvec": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
                                [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "qtip_gemm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
@@ -50,6 +52,9 @@ _SIGNATURES = {
     "qtip_rht_post_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_float, ctypes.c_void_p]),
+    "qtip_rht_fused_pre_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
+                                               ctypes.c_float, ctypes.c_void_p]),
     "qtip_rht_fused": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                       ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                       ctypes.c_void_p, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_float,

@@ -271,6 +271,7 @@ struct GroupArgs {
   const uint8_t* packed[3];
   const uint32_t* tlut[3];
   const uint16_t* su[3];
+  const uint16_t* x[3];       // the matrices' own inputs (plain form; unused with a layer boundary)
   int m[3];
   int wg_begin[4];
   int upw_q[3], upw_r[3];
@@ -391,12 +392,13 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 // made the 28672-wide matrices 15-20 % slower).
 template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false, bool GROUP = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
-    float* __restrict__ dst_, const uint8_t* __restrict__ packed_, const uint16_t* __restrict__ x,
+    float* __restrict__ dst_, const uint8_t* __restrict__ packed_, const uint16_t* __restrict__ x_,
     const uint32_t* __restrict__ tlut_, int m_, int k, int wl_per, int upw_q_, int upw_r_,
     const uint16_t* __restrict__ su_ = nullptr, float xscale = 1.f, const ChainArgs chain = ChainArgs{},
     const GroupArgs grp = GroupArgs{}) {
   static_assert(!XFORM || XLDS, "the transformed activations live in LDS");
-  static_assert(!GROUP || XFORM == 2, "grouped launches exist for the layer-boundary form");
+  static_assert(!GROUP || XFORM == 2 || (XFORM == 0 && XLDS && !XHALF),
+                "grouped launches exist for the layer-boundary form and the plain form with x in LDS");
   // the matrix this workgroup serves (uniform: scalar selects on kernel arguments)
   int gi = 0;
   if constexpr (GROUP) gi = (int)blockIdx.y >= grp.wg_begin[2] ? 2 : ((int)blockIdx.y >= grp.wg_begin[1] ? 1 : 0);
@@ -404,6 +406,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const uint8_t* __restrict__ packed = GROUP ? pick3(grp.packed, gi) : packed_;
   const uint32_t* __restrict__ tlut = GROUP ? pick3(grp.tlut, gi) : tlut_;
   const uint16_t* __restrict__ su = GROUP ? pick3(grp.su, gi) : su_;
+  const uint16_t* __restrict__ x = (GROUP && XFORM == 0) ? pick3(grp.x, gi) : x_;
   const int m = GROUP ? pick3(grp.m, gi) : m_;
   const int upw_q = GROUP ? pick3(grp.upw_q, gi) : upw_q_;
   const int upw_r = GROUP ? pick3(grp.upw_r, gi) : upw_r_;
@@ -1035,6 +1038,9 @@ hipError_t setup_once() {
     QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<2, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<3, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
+    QTIP_ALLOW((matvec_kernel<4, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<2, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<3, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
     QTIP_ALLOW((matvec_kernel<4, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
@@ -1105,7 +1111,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 14; }
+int qtip_abi_version(void) { return 15; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -1280,44 +1286,16 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
   return launch_matvec(parts, packed, su_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale_in, &c);
 }
 
-int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* const* packed,
-                                       const void* const* tlut, const void* const* su_f16, const int* m,
-                                       int k, int bits, int nparts, const float* prev_parts,
-                                       int prev_nparts, size_t prev_part_stride, const float* post,
-                                       float scale_out, const void* residual_f16, const void* norm_w_f16,
-                                       float eps, float scale_in, void* x_out_f16, void* stream) {
-  if (!parts || !packed || !tlut || !su_f16 || !m) return QTIP_E_NULL;
-  if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
-  long m_total = 0;
-  for (int g = 0; g < ngroups; ++g) {
-    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits);
-    if (rc) return rc;
-    if (!aligned16(su_f16[g])) return QTIP_E_ALIGN;
-    m_total += m[g];
-  }
-  if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
-  if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
-  if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
-  if (prev_nparts < 1 || prev_nparts > kMaxSplit || x_out_f16 == residual_f16) return QTIP_E_SHAPE;
-  if (!aligned16(prev_parts) || !aligned16(post) || !aligned16(residual_f16) || !aligned16(norm_w_f16) ||
-      !aligned16(x_out_f16) || ((prev_part_stride * sizeof(float)) & 15u))
-    return QTIP_E_ALIGN;
-  ChainArgs c;
-  c.parts = prev_parts;
-  c.post = post;
-  c.residual = (const _Float16*)residual_f16;
-  c.norm_w = (const _Float16*)norm_w_f16;
-  c.x_out = (_Float16*)x_out_f16;
-  c.part_stride = prev_part_stride;
-  c.scale_out = scale_out;
-  c.eps = eps;
-  c.in_parts = prev_nparts;
+}  // extern "C"
 
-  // workgroups per k range, shared out in proportion to the matrices' row blocks (at least one
-  // each, never more than a matrix has row blocks)
-  const int S = nparts;
+// Workgroups per k range shared out among the matrices of a grouped launch in proportion to
+// their row blocks (at least one each, never more than a matrix has row blocks); fills every
+// field of GroupArgs except the pointers' meaning-specific ones (su / x).  Returns the number of
+// workgroups per k range, 0 if the device is too small for the group.
+static int share_out_group(GroupArgs& ga, float* parts, int ngroups, const void* const* packed,
+                           const void* const* tlut, const int* m, int S, long m_total) {
   const int P = device_info().cus / S;
-  if (P < ngroups) return QTIP_E_SHAPE;
+  if (P < ngroups) return 0;
   int nrb[3] = {0, 0, 0}, wg[3] = {0, 0, 0};
   long nrb_total = 0;
   for (int g = 0; g < ngroups; ++g) {
@@ -1356,7 +1334,6 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
       grown = true;
     }
   }
-  GroupArgs ga;
   int begin = 0;
   long col = 0;
   for (int g = 0; g < 3; ++g) {
@@ -1364,7 +1341,8 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
     ga.dst[g] = parts + (g < ngroups ? col : 0);
     ga.packed[g] = (const uint8_t*)packed[gg];
     ga.tlut[g] = (const uint32_t*)tlut[gg];
-    ga.su[g] = (const uint16_t*)su_f16[gg];
+    ga.su[g] = nullptr;
+    ga.x[g] = nullptr;
     ga.m[g] = m[gg];
     ga.wg_begin[g] = g < ngroups ? begin : used;
     ga.upw_q[g] = g < ngroups ? nrb[g] / wg[g] : 0;
@@ -1376,6 +1354,49 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
   }
   ga.wg_begin[3] = used;
   ga.part_stride = (size_t)m_total;
+  return used;
+}
+
+extern "C" {
+
+int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* const* packed,
+                                       const void* const* tlut, const void* const* su_f16, const int* m,
+                                       int k, int bits, int nparts, const float* prev_parts,
+                                       int prev_nparts, size_t prev_part_stride, const float* post,
+                                       float scale_out, const void* residual_f16, const void* norm_w_f16,
+                                       float eps, float scale_in, void* x_out_f16, void* stream) {
+  if (!parts || !packed || !tlut || !su_f16 || !m) return QTIP_E_NULL;
+  if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
+  long m_total = 0;
+  for (int g = 0; g < ngroups; ++g) {
+    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits);
+    if (rc) return rc;
+    if (!aligned16(su_f16[g])) return QTIP_E_ALIGN;
+    m_total += m[g];
+  }
+  if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
+  if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
+  if (prev_nparts < 1 || prev_nparts > kMaxSplit || x_out_f16 == residual_f16) return QTIP_E_SHAPE;
+  if (!aligned16(prev_parts) || !aligned16(post) || !aligned16(residual_f16) || !aligned16(norm_w_f16) ||
+      !aligned16(x_out_f16) || ((prev_part_stride * sizeof(float)) & 15u))
+    return QTIP_E_ALIGN;
+  ChainArgs c;
+  c.parts = prev_parts;
+  c.post = post;
+  c.residual = (const _Float16*)residual_f16;
+  c.norm_w = (const _Float16*)norm_w_f16;
+  c.x_out = (_Float16*)x_out_f16;
+  c.part_stride = prev_part_stride;
+  c.scale_out = scale_out;
+  c.eps = eps;
+  c.in_parts = prev_nparts;
+
+  const int S = nparts;
+  GroupArgs ga;
+  const int used = share_out_group(ga, parts, ngroups, packed, tlut, m, S, m_total);
+  if (used == 0) return QTIP_E_SHAPE;
+  for (int g = 0; g < 3; ++g) ga.su[g] = (const uint16_t*)su_f16[g < ngroups ? g : ngroups - 1];
   const int nwl = ((k >> 5) + 3) >> 2;
   const int wl_per = (nwl + S - 1) / S;
   const dim3 g2((unsigned)S, (unsigned)used);
@@ -1385,6 +1406,39 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
     case 2: matvec_kernel<2, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
     case 3: matvec_kernel<3, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
     default: matvec_kernel<4, 2, true, 2, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, scale_in, c, ga); break;
+  }
+  return (int)hipGetLastError();
+}
+
+int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* packed,
+                                 const void* const* x_f16, const void* const* tlut, const int* m, int k,
+                                 int bits, int nparts, void* stream) {
+  if (!parts || !packed || !tlut || !x_f16 || !m) return QTIP_E_NULL;
+  if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
+  long m_total = 0;
+  for (int g = 0; g < ngroups; ++g) {
+    int rc = check_matvec(parts, packed[g], x_f16[g], tlut[g], m[g], k, bits);
+    if (rc) return rc;
+    if (!aligned16(x_f16[g])) return QTIP_E_ALIGN;
+    m_total += m[g];
+  }
+  const int nwl = ((k >> 5) + 3) >> 2;
+  if (nparts < 1 || nparts > kMaxSplit || nparts > nwl) return QTIP_E_SHAPE;
+  const int S = nparts;
+  const int wl_per = (nwl + S - 1) / S;
+  const size_t xbytes = (size_t)wl_per * 256;
+  if (xbytes > kMatvecXBytes) return QTIP_E_SHAPE;  // the grouped plain form keeps x in LDS
+  GroupArgs ga;
+  const int used = share_out_group(ga, parts, ngroups, packed, tlut, m, S, m_total);
+  if (used == 0) return QTIP_E_SHAPE;
+  for (int g = 0; g < 3; ++g) ga.x[g] = (const uint16_t*)x_f16[g < ngroups ? g : ngroups - 1];
+  const dim3 g2((unsigned)S, (unsigned)used);
+  const size_t lds = kMatvecLds + xbytes;
+  hipStream_t st = (hipStream_t)stream;
+  switch (bits) {
+    case 2: matvec_kernel<2, 2, true, 0, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, 1.f, ChainArgs{}, ga); break;
+    case 3: matvec_kernel<3, 2, true, 0, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, 1.f, ChainArgs{}, ga); break;
+    default: matvec_kernel<4, 2, true, 0, false, true><<<g2, kThreads, lds, st>>>(nullptr, nullptr, nullptr, nullptr, 0, k, wl_per, 0, 0, nullptr, 1.f, ChainArgs{}, ga); break;
   }
   return (int)hipGetLastError();
 }

@@ -42,6 +42,7 @@ struct RhtParams {
   size_t part_stride;
   size_t in_row_stride;      // elements between consecutive rows of `in`
   size_t post_row_stride;    // elements between the rows' `post` vectors (0: one vector for all rows)
+  size_t pre_row_stride;     // the same for `pre`
   float scale, eps;
   int in_parts, n, order, logA, pp, pre_mode;
   // from the host (divisions and search loops in the prologue of a latency-bound kernel are time on
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
     }
     if (P.pre) {
 #pragma unroll
-      for (int q = 0; q < CH; ++q) sr[q] = P.pre[idx[q]];
+      for (int q = 0; q < CH; ++q) sr[q] = P.pre[r * P.pre_row_stride + idx[q]];
     }
     if (order > 1) {
 #pragma unroll
@@ -325,7 +326,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
     }
     if (P.pre) {
 #pragma unroll
-      for (int q = 0; q < CH; ++q) sr[q].load(P.pre + base[q]);
+      for (int q = 0; q < CH; ++q) sr[q].load(P.pre + r * P.pre_row_stride + base[q]);
     }
     if (order > 1) {
 #pragma unroll
@@ -514,7 +515,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_rows_kernel(const RhtParams P
   if (P.post) ld_f32<EPT>(P.post + r * P.post_row_stride + e_swp, pv);
   if (P.pre) {
     float sv[EPT];
-    ld_f16<EPT>(P.pre + e_nat, sv);
+    ld_f16<EPT>(P.pre + r * P.pre_row_stride + e_nat, sv);
     for (int w = 1; w < P.in_parts; ++w) {
       float t[EPT];
       load(src + w * P.part_stride + e_nat, t);
@@ -814,6 +815,29 @@ int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int i
   P.order = order;
   P.pre_mode = pre_mode;
   return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+int qtip_rht_fused_pre_rows(void* out_f16, const void* in_f16, int rows, int n, int order,
+                            const uint32_t* had_bits, const void* pre_rows_f16, float scale,
+                            const void* norm_weight_f16, float eps, void* stream) {
+  if (!pre_rows_f16 || !norm_weight_f16) return QTIP_E_NULL;
+  if ((reinterpret_cast<uintptr_t>(pre_rows_f16) & 15u) || ((size_t)(n > 0 ? n : 0) * 2 & 15u)) return QTIP_E_ALIGN;
+  RhtParams P{};
+  P.out = out_f16;
+  P.in = in_f16;
+  P.had_bits = had_bits;
+  P.pre = (const _Float16*)pre_rows_f16;
+  P.pre_row_stride = (size_t)(n > 0 ? n : 0);
+  P.norm_w = (const _Float16*)norm_weight_f16;
+  P.part_stride = 0;
+  P.in_row_stride = 0;  // every row transforms the same input vector
+  P.scale = scale;
+  P.eps = eps;
+  P.in_parts = 1;
+  P.n = n;
+  P.order = order;
+  P.pre_mode = PRE_RMSNORM;
+  return launch_rht(P, QTIP_F16, QTIP_F16, rows, stream);
 }
 
 int qtip_rht_chain(void* xt_out_f16, void* x_out_f16, const float* parts, int in_parts, int rows, int n,

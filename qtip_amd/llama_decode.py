@@ -152,6 +152,8 @@ class DecoderLayer(nn.Module):
         f = self._fused_linears()
         if self.grouped_ok():
             return self._decode_grouped(x, k_cache, v_cache, pos, inv_freq, qkv_parts, next_layer)
+        if self.grouped_plain_ok():
+            return self._decode_grouped_plain(x, k_cache, v_cache, pos, inv_freq), None
         if self.fused:
             if qkv_parts is None:
                 qkv_parts = f['qkv'].matvec(f['qkv'].transform_in(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps))
@@ -208,6 +210,65 @@ class DecoderLayer(nn.Module):
                         self._sv_gate_up = torch.stack([g.SV, u.SV]).contiguous()
             self._grouped = ok
         return self._grouped
+
+    def grouped_plain_ok(self):
+        """Separate projections whose hidden size is not one the matvec transforms itself (e.g.
+        5120 = 40 x 128): the transforms stay launches of their own, but the projections that
+        share an input still share their launches."""
+        if not hasattr(self, "_grouped_plain"):
+            ok = not self.fused and not self.grouped_ok()
+            if ok:
+                f = self._fused_linears()
+                cfg = self.cfg
+                ok = not any(l.dense for l in f.values())
+                if ok:
+                    q, k, v, g, u = (f[n] for n in ('q_proj', 'k_proj', 'v_proj', 'gate_proj', 'up_proj'))
+                    ok = (q.K == k.K == v.K and g.K == u.K and g.m == u.m and g.Kr == u.Kr
+                          and all(l.n == cfg.hidden and l.Kl == q.Kl for l in (q, k, v, g, u))
+                          and all(l.out_transform_fits_attention(cfg.head_dim) for l in (q, k, v))
+                          and all(l.SU.dtype == torch.float16 for l in (q, k, v, g, u))
+                          and cfg.hidden * 2 <= 28 * 1024)
+                    if ok:
+                        self._sv_gate_up = torch.stack([g.SV, u.SV]).contiguous()
+                        self._su_qkv = torch.stack([q.SU, k.SU, v.SU]).contiguous()
+                        self._su_gate_up = torch.stack([g.SU, u.SU]).contiguous()
+            self._grouped_plain = ok
+        return self._grouped_plain
+
+    def _group_plain(self, names, x, su_rows, norm_weight):
+        """Two launches: the input transforms (RMSNorm, one sign vector per projection) and the
+        matvecs of the projections `names`, which read the same vector."""
+        f = self._fused_linears()
+        ls = [f[n] for n in names]
+        l0 = ls[0]
+        xt = ops.rht_fused_pre_rows(x, su_rows, norm_weight, self.cfg.eps, order=l0.Kl, had_bits=l0.bl,
+                                    scale=(l0.n**-0.5) / 32.0)
+        return ops.decompress_matvec_group([l.trellis for l in ls], [xt[i] for i in range(len(ls))],
+                                           [l.tlut for l in ls], [l.m for l in ls], l0.n, l0.K)
+
+    def _decode_grouped_plain(self, x, k_cache, v_cache, pos, inv_freq):
+        """decode_fused for separate projections with a hidden size the matvec does not transform
+        itself, 12 launches: [RMSNorm + three input transforms], [q, k, v matvecs], attention with
+        the three output transforms in its prologue, o as transform / matvec / transform +
+        residual, [RMSNorm + two input transforms], [gate, up matvecs], both output transforms,
+        and down as [SiLU * up + transform] / matvec / transform + residual."""
+        cfg = self.cfg
+        f = self._fused_linears()
+        qkv = [f[n] for n in ('q_proj', 'k_proj', 'v_proj')]
+        qkv_parts = self._group_plain(('q_proj', 'k_proj', 'v_proj'), x, self._su_qkv, self.input_norm.weight)
+        views, off = [], 0
+        for l in qkv:
+            views.append(qkv_parts[:, off:off + l.m])
+            off += l.m
+        attn = ops.decode_attention_rht3(views, [l.SV for l in qkv], [(l.m**-0.5) * 32.0 for l in qkv],
+                                         [l.br for l in qkv], [l.Kr for l in qkv], k_cache, v_cache, pos, inv_freq,
+                                         cfg.heads, cfg.kv_heads, cfg.head_dim)
+        x = f['o'](attn.reshape(1, -1), residual=x)
+        gu_parts = self._group_plain(('gate_proj', 'up_proj'), x, self._su_gate_up, self.post_norm.weight)
+        g = f['gate_proj']
+        ug = ops.rht_post_rows(gu_parts.view(gu_parts.shape[0], 2, g.m), self._sv_gate_up, order=g.Kr, had_bits=g.br,
+                               scale=(g.m**-0.5) * 32.0)
+        return f['down'](ug.reshape(1, -1), ops.PRE_SILU_MUL, residual=x)
 
     def _group_chain(self, names, prev_parts, prev, residual, norm_weight):
         """One launch: boundary after `prev` (its output transform, residual, RMSNorm) and the

@@ -212,6 +212,30 @@ def decompress_matvec_group_chain(packed, tlut, m, k, bits, prev_parts, post, sc
     return parts, x_new
 
 
+def decompress_matvec_group(packed, x, tlut, m, k, bits, nparts=None):
+    """Up to three matvecs of the same k and bit width in one launch, matrix g on its own fp16
+    input x[g] (k values each; rows of one tensor will do).  Returns parts (S, sum(m)) fp32."""
+    n = len(packed)
+    if not (1 <= n <= 3) or len(tlut) != n or len(m) != n or len(x) != n:
+        raise ValueError("one to three matrices, with one table, row count and input each")
+    dev = packed[0].device
+    for g in range(n):
+        _check_packed(packed[g], m[g], k, bits)
+        _check_tlut(tlut[g], dev)
+        require_cuda(x[g], "x", torch.float16)
+        if x[g].numel() != k or x[g].device != dev or packed[g].device != dev:
+            raise ValueError(f"every x must hold k = {k} values on {dev}")
+    m_total = int(sum(m))
+    S = int(nparts) if nparts is not None else matvec_split(m_total, k, bits, dev)
+    parts = torch.empty((S, m_total), dtype=torch.float32, device=dev)
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+    with torch.cuda.device(dev):
+        check(lib().qtip_decompress_matvec_group(_ptr(parts), n, ptrs(packed), ptrs(x), ptrs(tlut),
+                                                 (ctypes.c_int * n)(*[int(v) for v in m]), k, bits, S,
+                                                 stream_ptr(dev)), "qtip_decompress_matvec_group")
+    return parts
+
+
 def decompress_gemm(packed, x, tlut, m, k, bits, round_f16=True):
     """(batch, m) fp32 = x[batch,k] (fp16) @ decode(packed)[m,k]^T on the matrix cores."""
     _check_packed(packed, m, k, bits)
@@ -315,6 +339,29 @@ def rht(x, order=1, had_bits=None, pre=None, post=None, scale=None, out_dtype=No
                 check(L.qtip_rht(_ptr(of[r0:r1]), _DT[out_dtype], _ptr(src), _DT[x.dtype], in_parts, r1 - r0, n,
                                  order, _ptr(had_bits), _ptr(pre), _ptr(post), ctypes.c_float(scale),
                                  stream_ptr(x.device)), "qtip_rht")
+    return out
+
+
+def rht_fused_pre_rows(x, pre_rows, norm_weight, eps, order=1, had_bits=None, scale=None):
+    """Input transforms of `rows` layers that read the same fp16 vector x (n values), one launch:
+    row r = fp16(scale * H^T(pre_rows[r] * rmsnorm(x))).  pre_rows (rows, n) fp16.  -> (rows, n)."""
+    require_cuda(x, "x", torch.float16)
+    require_cuda(pre_rows, "pre_rows", torch.float16)
+    require_cuda(norm_weight, "norm_weight", torch.float16)
+    n = x.numel()
+    if pre_rows.dim() != 2 or pre_rows.shape[1] != n or norm_weight.numel() != n or pre_rows.shape[0] > 65535:
+        raise ValueError("pre_rows must be (rows, n) and norm_weight hold n values")
+    p = n // order
+    if n % order or p & (p - 1):
+        raise ValueError(f"{n} is not {order} times a power of two")
+    if order > 1:
+        require_cuda(had_bits, "had_bits", torch.int32)
+    out = torch.empty_like(pre_rows)
+    with torch.cuda.device(x.device):
+        check(lib().qtip_rht_fused_pre_rows(_ptr(out), _ptr(x), pre_rows.shape[0], n, order, _ptr(had_bits),
+                                            _ptr(pre_rows), ctypes.c_float(scale if scale is not None else n ** -0.5),
+                                            _ptr(norm_weight), ctypes.c_float(eps), stream_ptr(x.device)),
+              "qtip_rht_fused_pre_rows")
     return out
 
 

@@ -634,6 +634,27 @@ def test_decode_of_separate_projections_in_grouped_launches(heads, kv_heads):
     assert torch.equal(out, ref)
 
 
+def test_decode_of_separate_projections_with_a_table_order_hidden_size():
+    """Hidden size 40 x 64 (the 13B kind: a table order times a power of two): the projections
+    that share an input share their launches (12 per layer); logits and caches of the
+    module-by-module forward."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder
+    cfg = LlamaConfig(hidden=2560, heads=20, kv_heads=20, layers=2, ffn=108 * 32, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64, fused=False)
+    assert all(layer.grouped_plain_ok() and not layer.grouped_ok() for layer in model.layers)
+    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(5, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([5], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        b = model.decode_fused(tok, pos)
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    for c0, c1 in zip(kc, model.k_cache):
+        assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+
+
 def test_generate_falls_back_for_per_shard_transforms():
     """A model quantised with per-shard transforms (rcp != 0) is outside the fused decode step:
     generate() decodes it module by module instead of failing."""
@@ -814,6 +835,45 @@ def test_grouped_matvec_with_layer_boundary(K, ms, k, S, Sp):
         assert torch.equal(x_one, x_new)
         assert torch.equal(parts[:, off:off + m], one), (i, m)
         off += m
+
+
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("ms,k,S", [((512, 512, 512), 5120, None), ((5120, 5120, 5120), 5120, 2), ((13824, 13824), 5120, 1),
+                                    ((64,), 1024, 1), ((32, 96, 2048), 11008, 2)])
+def test_grouped_plain_matvec(K, ms, k, S):
+    """Up to three matrices, each on its own input, in one launch: bit-identical to the
+    single-matrix launches."""
+    from qtip_amd import ops
+    if K != 2 and sum(ms) > 16384:
+        pytest.skip("large shapes once")
+    layers = [make_layer(m, k, K, seed=m + k + K + 7 * i) for i, m in enumerate(ms)]
+    packed = [dev(L["packed"]).reshape(-1) for L in layers]
+    tluts = [dev(L["tlut"]).reshape(-1) for L in layers]
+    xs = torch.randn(len(ms), k, generator=torch.Generator().manual_seed(k + K)).half().cuda()
+    parts = ops.decompress_matvec_group(packed, [xs[i] for i in range(len(ms))], tluts, list(ms), k, K, nparts=S)
+    off = 0
+    for i, m in enumerate(ms):
+        one = ops.decompress_matvec_parts(packed[i], xs[i], tluts[i], m, k, K, nparts=parts.shape[0])
+        assert torch.equal(parts[:, off:off + m], one.reshape(parts.shape[0], m)), (i, m)
+        off += m
+
+
+@pytest.mark.parametrize("n", [5120, 4096, 1024, 11008, 13824])
+def test_input_transforms_of_several_layers_in_one_launch(n):
+    """rht_fused_pre_rows == one fused RMSNorm + transform launch per sign vector, bit for bit."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(1, n, generator=g).half().cuda()
+    w = (1 + 0.1 * torch.randn(n, generator=g)).half().cuda()
+    pre = torch.sign(torch.randn(3, n, generator=g) + 1e-5).half().cuda()
+    hadK, order = get_hadK(n)
+    bits = had_bits(hadK, order, True, "cuda") if order > 1 else None
+    got = ops.rht_fused_pre_rows(x, pre, w, 1e-5, order=order, had_bits=bits, scale=n**-0.5 / 32)
+    for r in range(3):
+        one = ops.rht(x, order=order, had_bits=bits, pre=pre[r].contiguous(), scale=n**-0.5 / 32,
+                      out_dtype=torch.float16, pre_mode=ops.PRE_RMSNORM, norm_weight=w, eps=1e-5)
+        assert torch.equal(got[r], one.reshape(-1)), (n, r)
 
 
 def test_forward_many_rows_decodes_and_multiplies():
