@@ -226,8 +226,7 @@ class DecoderLayer(nn.Module):
                     ok = (q.K == k.K == v.K and g.K == u.K and g.m == u.m and g.Kr == u.Kr
                           and all(l.n == cfg.hidden and l.Kl == q.Kl for l in (q, k, v, g, u))
                           and all(l.out_transform_fits_attention(cfg.head_dim) for l in (q, k, v))
-                          and all(l.SU.dtype == torch.float16 for l in (q, k, v, g, u))
-                          and cfg.hidden * 2 <= 28 * 1024)
+                          and all(l.SU.dtype == torch.float16 for l in (q, k, v, g, u)))
                     if ok:
                         self._sv_gate_up = torch.stack([g.SV, u.SV]).contiguous()
                         self._su_qkv = torch.stack([q.SU, k.SU, v.SU]).contiguous()

@@ -226,7 +226,12 @@ def decompress_matvec_group(packed, x, tlut, m, k, bits, nparts=None):
         if x[g].numel() != k or x[g].device != dev or packed[g].device != dev:
             raise ValueError(f"every x must hold k = {k} values on {dev}")
     m_total = int(sum(m))
-    S = int(nparts) if nparts is not None else matvec_split(m_total, k, bits, dev)
+    if nparts is not None:
+        S = int(nparts)
+    else:
+        S = matvec_split(m_total, k, bits, dev)
+        while k * 2 > S * 28 * 1024:  # every k range of x has to fit the kernel's staging area
+            S *= 2
     parts = torch.empty((S, m_total), dtype=torch.float32, device=dev)
     ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
     with torch.cuda.device(dev):
