@@ -271,6 +271,17 @@ int qtip_rmsnorm(void* out_f16, const void* x_f16, const void* weight_f16, float
 int qtip_greedy_pick(const void* logits_f16, int vocab, void* tok_i64, void* pos_i64, void* history_i64,
                      long history_len, long history_base, void* stream);
 
+/* Sampled token pick of the generation loop (eval/interactive_gen.py:15-40: logits / max(temperature,
+ * 1e-5), entries below the top_k-th largest logit removed, softmax, a draw by the exponential race
+ * argmax(p / q), q ~ Exp(1)) with the bookkeeping of qtip_greedy_pick, one launch.  top_k 0 keeps
+ * the whole vocabulary, at most 64.  The race is evaluated as argmax(logit / T - log q) with q from
+ * a counter-based generator keyed by (seed, counter_i64[0], entry); the counter is device memory
+ * and advances by one per launch, so a recorded graph draws fresh numbers at every replay.  The
+ * distribution is the reference's; the random stream is this library's own. */
+int qtip_sample_pick(const void* logits_f16, int vocab, float temperature, int top_k, unsigned seed,
+                     void* counter_i64, void* tok_i64, void* pos_i64, void* history_i64, long history_len,
+                     long history_base, void* stream);
+
 /* Measurement aid, no counterpart in the reference: reads `bytes` of device memory once with the
  * matvec's kind of loads (persistent workgroups, one non-temporal 16-byte load per lane) and
  * writes one folded word per wave to sink_u32 (16 * #CUs words).  Its duration is the stream-read

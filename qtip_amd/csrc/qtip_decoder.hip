@@ -656,3 +656,125 @@ extern "C" int qtip_greedy_pick(const void* logits_f16, int vocab, void* tok_i64
                                                                  history_base);
   return (int)hipGetLastError();
 }
+
+// ---- sampled token pick ----------------------------------------------------------------------
+
+namespace {
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+// (value, index) pairs ordered by value descending, index ascending; `before(a, b)`: a comes first
+__device__ __forceinline__ bool before(float av, int ai, float bv, int bi) {
+  return av > bv || (av == bv && ai < bi);
+}
+
+// Sampling of eval/interactive_gen.py:15-40 in one launch: logits / temperature, everything below
+// the top_k-th largest logit removed (ties with it stay, as torch.where(logits < kth, -inf, logits)
+// keeps them), softmax, and a draw by the exponential race argmax(p_i / q_i), q_i ~ Exp(1) - which
+// is argmax(logit_i / T - log q_i).  The q_i come from a counter-based generator keyed by (seed,
+// draw counter, i); the counter lives in device memory and advances with every launch, so a
+// recorded graph draws fresh numbers at every replay.  Bookkeeping as in greedy_pick_kernel.
+__global__ __launch_bounds__(kHeadThreads) void sample_pick_kernel(const _Float16* __restrict__ logits, int vocab,
+                                                                   float inv_temperature, int top_k, uint32_t seed,
+                                                                   long* __restrict__ counter, long* __restrict__ tok,
+                                                                   long* __restrict__ pos, long* __restrict__ hist,
+                                                                   long hist_len, long hist_base) {
+  __shared__ float bv[16];
+  __shared__ int bi[16];
+  __shared__ float sel_v;
+  __shared__ int sel_i;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // block-wide first element in (value desc, index asc) order among those after (pv, pi)
+  auto next_after = [&](float pv, int pi, auto&& score) {
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = tid; i < vocab; i += kHeadThreads) {
+      const float raw = (float)logits[i];
+      if (before(pv, pi, raw, i)) {  // strictly after the previous pick
+        const float f = score(raw, i);
+        if (before(f, i, best, idx)) {
+          best = f;
+          idx = i;
+        }
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float ob = __shfl_xor(best, o);
+      const int oi = __shfl_xor(idx, o);
+      if (before(ob, oi, best, idx)) {
+        best = ob;
+        idx = oi;
+      }
+    }
+    __syncthreads();  // the previous round's result has been read by everyone
+    if (lane == 0) {
+      bv[wave] = best;
+      bi[wave] = idx;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      for (int q = 1; q < 16; ++q)
+        if (before(bv[q], bi[q], best, idx)) {
+          best = bv[q];
+          idx = bi[q];
+        }
+      sel_v = best;
+      sel_i = idx;
+    }
+    __syncthreads();
+  };
+  // ---- the top_k-th largest logit (with multiplicity): top_k rounds of "next in order"
+  float kth = -INFINITY;
+  if (top_k > 0 && top_k < vocab) {
+    float pv = INFINITY;
+    int pi = -1;
+    for (int r = 0; r < top_k; ++r) {
+      next_after(pv, pi, [](float raw, int) { return raw; });
+      pv = sel_v;
+      pi = sel_i;
+    }
+    kth = pv;
+  }
+  // ---- the race: argmax over the kept entries of logit / T - log(q), q = -log(u)
+  const uint32_t draw = (uint32_t)counter[0];
+  const uint32_t key = mix32(seed ^ mix32(draw + 0x9e3779b9U));
+  next_after(INFINITY, -1, [&](float raw, int i) {
+    if (raw < kth) return -INFINITY;
+    const uint32_t h = mix32(key ^ mix32((uint32_t)i * 0x85ebca6bU + 1u));
+    const float u = ((float)(h >> 8) + 0.5f) * (1.0f / 16777216.0f);  // (0, 1)
+    return raw * inv_temperature - __logf(-__logf(u));
+  });
+  if (tid == 0) {
+    int idx = sel_i;
+    if (idx == 0x7fffffff) idx = 0;
+    const long p = pos[0];
+    const long slot = p - hist_base;
+    if (hist && slot >= 0 && slot < hist_len) hist[slot] = idx;
+    tok[0] = idx;
+    pos[0] = p + 1;
+    counter[0] = (long)draw + 1;
+  }
+}
+
+}  // namespace
+
+extern "C" int qtip_sample_pick(const void* logits_f16, int vocab, float temperature, int top_k,
+                                unsigned seed, void* counter_i64, void* tok_i64, void* pos_i64,
+                                void* history_i64, long history_len, long history_base, void* stream) {
+  if (!logits_f16 || !counter_i64 || !tok_i64 || !pos_i64) return QTIP_E_NULL;
+  if (vocab < 1 || history_len < 0 || top_k < 0 || top_k > 64) return QTIP_E_SHAPE;
+  const float t = temperature > 1e-5f ? temperature : 1e-5f;  // max(temperature, 1e-5) as the reference
+  sample_pick_kernel<<<1, kHeadThreads, 0, (hipStream_t)stream>>>((const _Float16*)logits_f16, vocab, 1.0f / t, top_k,
+                                                                 seed, (long*)counter_i64, (long*)tok_i64,
+                                                                 (long*)pos_i64, (long*)history_i64, history_len,
+                                                                 history_base);
+  return (int)hipGetLastError();
+}

@@ -519,10 +519,13 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
     tok = pick(logits)
     static_tok = tok.clone()
     static_pos = torch.tensor([n], device=dev)
-    # greedy decoding on the fused kernels keeps its bookkeeping on the device: the pick kernel
-    # writes the next input token, the history slot and the advanced position, so a step is one
-    # graph replay and nothing else
-    on_device = fused and not sampling
+    # decoding on the fused kernels keeps its bookkeeping on the device: the pick kernel (greedy, or
+    # the sampled draw with its counter-based random numbers) writes the next input token, the
+    # history slot and the advanced position, so a step is one graph replay and nothing else
+    device_sampling = sampling and (top_k is None or top_k <= ops.SAMPLE_PICK_MAX_TOP_K)
+    on_device = fused and (not sampling or device_sampling)
+    seed = int(torch.randint(0, 2**31 - 1, (1,)).item()) if sampling else 0  # follows torch.manual_seed
+    draw_counter = torch.zeros(1, dtype=torch.int64, device=dev)
     history = torch.zeros(max(max_new_tokens, 1), dtype=torch.int64, device=dev)
     history[0] = tok.reshape(-1)[0]
     out = [tok.clone()]
@@ -530,17 +533,21 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
         callback(out[-1])
 
     def step():
-        # the random draw stays outside the captured graph: a replay would repeat it
+        # (a draw by the framework's generator stays outside the captured graph: a replay would repeat it)
         if on_device:
             lg = model.decode_fused(static_tok, static_pos, float_logits=False)
-            ops.greedy_pick(lg.reshape(-1), static_tok, static_pos, history, n - 1)
+            if sampling:
+                ops.sample_pick(lg.reshape(-1), temperature, top_k, seed, draw_counter, static_tok, static_pos,
+                                history, n - 1)
+            else:
+                ops.greedy_pick(lg.reshape(-1), static_tok, static_pos, history, n - 1)
             return None
         lg = model.decode_fused(static_tok, static_pos) if fused else model(static_tok, static_pos)
         return lg if sampling else pick(lg)
 
     graph = None
     if use_graph:
-        keep = (static_tok.clone(), static_pos.clone(), history.clone())
+        keep = (static_tok.clone(), static_pos.clone(), history.clone(), draw_counter.clone())
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
@@ -550,6 +557,7 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
                     static_tok.copy_(keep[0])
                     static_pos.copy_(keep[1])
                     history.copy_(keep[2])
+                    draw_counter.copy_(keep[3])
         torch.cuda.current_stream().wait_stream(s)
         # the warm-up wrote cache slot n with this token's k/v, which the timed step rewrites identically
         graph = torch.cuda.CUDAGraph()
@@ -559,6 +567,7 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
             static_tok.copy_(keep[0])
             static_pos.copy_(keep[1])
             history.copy_(keep[2])
+            draw_counter.copy_(keep[3])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(max_new_tokens - 1):

@@ -524,6 +524,30 @@ def probe_stream_read(src):
     return sink
 
 
+SAMPLE_PICK_MAX_TOP_K = 64
+
+
+def sample_pick(logits, temperature, top_k, seed, counter, tok, pos, history=None, history_base=0):
+    """Draw tok[0] from softmax(logits / temperature) restricted to the top_k largest logits
+    (None: all), as eval/interactive_gen.py:15-40 does, with the bookkeeping of greedy_pick, in
+    one launch.  counter: device int64 draw counter (advanced in place); seed: host integer."""
+    require_cuda(logits, "logits", torch.float16)
+    require_cuda(tok, "tok", torch.int64)
+    require_cuda(pos, "pos", torch.int64)
+    require_cuda(counter, "counter", torch.int64)
+    if history is not None:
+        require_cuda(history, "history", torch.int64)
+    k = 0 if top_k is None else int(top_k)
+    if tok.numel() != 1 or pos.numel() != 1 or counter.numel() != 1 or not (0 <= k <= SAMPLE_PICK_MAX_TOP_K):
+        raise ValueError("sample_pick: tok, pos and counter hold one element each, top_k at most 64")
+    with torch.cuda.device(logits.device):
+        check(lib().qtip_sample_pick(_ptr(logits), logits.numel(), ctypes.c_float(temperature), k,
+                                     ctypes.c_uint(int(seed) & 0xffffffff), _ptr(counter), _ptr(tok), _ptr(pos),
+                                     _ptr(history) if history is not None else None,
+                                     history.numel() if history is not None else 0, int(history_base),
+                                     stream_ptr(logits.device)), "qtip_sample_pick")
+
+
 # ---- packing tools ---------------------------------------------------------------------------
 
 def repack(packed, m, k, bits, to_kernel=True):

@@ -670,6 +670,48 @@ def test_generate_falls_back_for_per_shard_transforms():
     assert out.shape == (1, 5)
 
 
+def test_sample_pick_draws_from_the_reference_distribution():
+    """Sampled pick (eval/interactive_gen.py:15-40): top_k = 1 is the argmax; draws stay inside the
+    top-k set (ties with the k-th value included); empirical frequencies over 4000 draws follow
+    softmax(logits / T) on that set; the counter advances so replays differ."""
+    from qtip_amd import ops
+    g = torch.Generator().manual_seed(5)
+    vocab = 32003
+    lg = (torch.randn(vocab, generator=g) * 0.5).half()
+    top = [17, 4000, 31999, 12345, 9]
+    vals = [4.0, 3.5, 3.5, 3.0, 2.0]
+    for i, v in zip(top, vals):
+        lg[i] = v
+    lg = lg.cuda()
+    tok = torch.tensor([[0]], device="cuda")
+    pos = torch.tensor([10], device="cuda")
+    ctr = torch.zeros(1, dtype=torch.int64, device="cuda")
+    hist = torch.full((4,), -1, dtype=torch.int64, device="cuda")
+    ops.sample_pick(lg, 0.6, 1, 123, ctr, tok, pos, hist, 9)
+    assert int(tok) == 17 and int(pos) == 11 and int(ctr) == 1 and hist.tolist() == [-1, 17, -1, -1]
+    T, k, n = 0.8, 4, 4000
+    counts = {}
+    for _ in range(n):
+        ops.sample_pick(lg, T, k, 123, ctr, tok, pos)
+        t = int(tok)
+        counts[t] = counts.get(t, 0) + 1
+    assert int(ctr) == n + 1
+    assert set(counts) <= set(top[:4])  # the 4th largest value is 3.0; 2.0 is out
+    p = torch.softmax(torch.tensor(vals[:4]) / T, 0)
+    for i, pi in zip(top[:4], p.tolist()):
+        assert abs(counts.get(i, 0) / n - pi) < 0.03, (i, counts.get(i, 0) / n, pi)
+    # ties with the k-th value stay in: top_k = 2 keeps both 3.5 entries
+    counts = {}
+    for _ in range(600):
+        ops.sample_pick(lg, T, 2, 7, ctr, tok, pos)
+        counts[int(tok)] = counts.get(int(tok), 0) + 1
+    assert set(counts) == {17, 4000, 31999}
+    # the whole vocabulary (top_k None) at a low temperature: mostly the largest entries, never an error
+    for _ in range(50):
+        ops.sample_pick(lg, 0.05, None, 7, ctr, tok, pos)
+        assert int(tok) in (17, 4000, 31999)
+
+
 def test_generate_greedy_keeps_its_bookkeeping_on_the_device():
     """Greedy decoding through the captured step (pick kernel inside the graph) returns the tokens
     of the eager loop, and the streaming callback sees them in order."""
@@ -701,6 +743,10 @@ def test_generate_sampling_and_streaming():
     torch.manual_seed(5)
     drawn, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 8, temperature=0.6, top_k=5)
     assert drawn.shape == (1, 8) and int(drawn.min()) >= 0 and int(drawn.max()) < cfg.vocab
+    # the draw follows torch.manual_seed, with or without the captured graph
+    torch.manual_seed(5)
+    again, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64), ids, 8, temperature=0.6, top_k=5, use_graph=False)
+    assert torch.equal(drawn, again)
 
 
 def test_fused_decode_step_matches_generic():
