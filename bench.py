@@ -53,7 +53,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
     ap.add_argument("--extras", default="shapes,layer,gemm,decode,ceilings,e2e",
-                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, ceilings, e2e, e2e70b "
+                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, ceilings, e2e, e2e13b, e2e70b "
                          "(counter runs under rocprofv3 pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
@@ -309,6 +309,19 @@ def main():
         prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
         _, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
         result["e2e_decode_70b"] = {"model": "Llama-2-70B architecture, random init, 2-bit HYB, fused qkv and up/gate",
+                                    "prompt": 128, "new_tokens": 128, "tok_per_s": round(tps, 1),
+                                    "ms_per_token": round(1e3 / tps, 3)}
+        del model
+        torch.cuda.empty_cache()
+
+    if "e2e13b" in extras:
+        # a hidden size that is a table order times a power of two (5120 = 40 x 128), separate projections
+        from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+        cfg13 = LlamaConfig(hidden=5120, heads=40, kv_heads=40, layers=40, ffn=13824, vocab=32000, K=2)
+        model = LlamaDecoder(cfg13, max_cache_len=512, device=dev, fused=False)
+        prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
+        _, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
+        result["e2e_decode_13b"] = {"model": "Llama-2-13B architecture, random init, 2-bit HYB, separate projections",
                                     "prompt": 128, "new_tokens": 128, "tok_per_s": round(tps, 1),
                                     "ms_per_token": round(1e3 / tps, 3)}
         del model
