@@ -142,9 +142,11 @@ def main():
     # clock settling: the chip reaches its sustained clocks only after tens of milliseconds of
     # continuous work (a 3 ms timed region reads 10-15 % slower than a 40 ms one), so the timed
     # graph is replayed untimed until `settle_ms` of GPU time have passed, then timed once
+    before_settling = None
     if args.settle_ms > 0:
         torch.cuda.synchronize()
         one = timed(graph)
+        before_settling = one * 1e3 / args.steps
         for _ in range(min(1000, int(args.settle_ms * 1e-3 / max(one, 1e-6)))):
             graph.replay()
     torch.cuda.synchronize()
@@ -178,6 +180,7 @@ def main():
             "weight_copies_rotated": copies,
             "timing": "one HIP graph holding all timed steps, HIP events on the launch stream",
             "clock_settle_ms": args.settle_ms,
+            "ms_per_step_before_settling": round(before_settling, 5) if before_settling is not None else None,
         },
         "roofline": {
             "bound": "hbm",
