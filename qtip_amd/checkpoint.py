@@ -79,7 +79,7 @@ def read_config(path):
     cfg = LlamaConfig(hidden=c['hidden_size'], heads=heads, kv_heads=c.get('num_key_value_heads', heads),
                       layers=c['num_hidden_layers'], ffn=c['intermediate_size'], vocab=c['vocab_size'],
                       rope_theta=float(c.get('rope_theta', 10000.0)), eps=float(c.get('rms_norm_eps', 1e-5)),
-                      K=qp['K'])
+                      K=qp['K'], rope_scaling=c.get('rope_scaling'))
     return cfg, qp
 
 
@@ -163,6 +163,8 @@ def save_llama(model, path, max_shard_bytes=4 << 30):
                   hidden_act='silu', torch_dtype='float16',
                   quip_params=dict(td_x=16, td_y=16, L=16, K=cfg.K, V=2, tlut_bits=9, decode_mode='quantlut_sym',
                                    skip_list=skip))
+    if cfg.rope_scaling:
+        config['rope_scaling'] = cfg.rope_scaling
     kv = [l.v_proj.K for l in model.layers if isinstance(l.v_proj, QuantizedLinear)]
     if kv and kv[0] != cfg.K:
         config['quip_params']['K_v_proj'] = kv[0]

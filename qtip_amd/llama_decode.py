@@ -29,10 +29,37 @@ from .utils.matmul_had import had_bits
 class LlamaConfig:
 
     def __init__(self, hidden=4096, heads=32, kv_heads=32, layers=32, ffn=11008, vocab=32000, rope_theta=10000.0,
-                 eps=1e-5, K=2):
+                 eps=1e-5, K=2, rope_scaling=None):
         self.hidden, self.heads, self.kv_heads, self.layers = hidden, heads, kv_heads, layers
         self.ffn, self.vocab, self.rope_theta, self.eps, self.K = ffn, vocab, rope_theta, eps, K
         self.head_dim = hidden // heads
+        self.rope_scaling = dict(rope_scaling) if rope_scaling else None
+
+
+def rope_inv_freq(cfg):
+    """Rotary frequencies of the model, fp32 (head_dim / 2,).  `rope_scaling` as in the Hugging Face
+    config the reference's LlamaRotaryEmbedding reads (model/llama.py:150-190): none / "default",
+    "linear" (frequencies divided by the factor) and "llama3" (the Llama-3.1 rule: long wavelengths
+    divided by the factor, a smooth blend in the band between the two wavelength limits).  The types
+    that change with the sequence length ("dynamic", ...) are not supported by the static tables of
+    the decode loop."""
+    inv_freq = 1.0 / (cfg.rope_theta**(torch.arange(0, cfg.head_dim, 2, dtype=torch.float32) / cfg.head_dim))
+    rs = cfg.rope_scaling
+    kind = (rs.get("rope_type", rs.get("type")) if rs else None) or "default"
+    if kind == "default":
+        return inv_freq
+    if kind == "linear":
+        return inv_freq / float(rs["factor"])
+    if kind == "llama3":
+        factor, lo, hi = float(rs["factor"]), float(rs["low_freq_factor"]), float(rs["high_freq_factor"])
+        old_len = float(rs["original_max_position_embeddings"])
+        wavelen = 2 * math.pi / inv_freq
+        scaled = torch.where(wavelen > old_len / lo, inv_freq / factor, inv_freq)
+        smooth = (old_len / wavelen - lo) / (hi - lo)
+        blended = (1 - smooth) * scaled / factor + smooth * scaled
+        medium = ~(wavelen < old_len / hi) & ~(wavelen > old_len / lo)
+        return torch.where(medium, blended, scaled)
+    raise NotImplementedError(f"rope_scaling type {kind!r}")
 
 
 def _qlinear(cfg, fin, fout, gen, device, K=None):
@@ -432,8 +459,7 @@ class LlamaDecoder(nn.Module):
         shape = (1, cfg.kv_heads, max_cache_len, cfg.head_dim)
         self.k_cache = [torch.zeros(shape, dtype=torch.float16, device=device) for _ in range(cfg.layers)]
         self.v_cache = [torch.zeros(shape, dtype=torch.float16, device=device) for _ in range(cfg.layers)]
-        inv_freq = 1.0 / (cfg.rope_theta**(torch.arange(0, cfg.head_dim, 2, dtype=torch.float32) / cfg.head_dim))
-        self.inv_freq = inv_freq.to(device)
+        self.inv_freq = rope_inv_freq(cfg).to(device)
 
     def rope(self, positions):
         freqs = positions.float()[:, None] * self.inv_freq[None, :]

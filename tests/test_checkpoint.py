@@ -26,6 +26,9 @@ def _state(model):
 @pytest.mark.parametrize("shard_bytes", [4 << 30, 100000])
 def test_save_load_round_trip_cpu(tmp_path, shard_bytes):
     model = _tiny('cpu', K_v=3)
+    l3 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+    model.cfg.rope_scaling = dict(l3)
     for layer in model.layers:  # skipped projections and norms get non-trivial values
         layer.input_norm.weight.data.uniform_(0.5, 1.5)
         for mod in layer.children():
@@ -39,6 +42,9 @@ def test_save_load_round_trip_cpu(tmp_path, shard_bytes):
     cfg = json.load(open(tmp_path / 'config.json'))
     assert cfg['quip_params']['skip_list'] == ['0_down', '1_k'] and cfg['quip_params']['K_v_proj'] == 3
     loaded = C.load_llama(str(tmp_path), max_cache_len=64, device='cpu')
+    assert cfg['rope_scaling'] == l3 and loaded.cfg.rope_scaling == l3
+    from qtip_amd.llama_decode import rope_inv_freq
+    assert torch.equal(loaded.inv_freq, rope_inv_freq(loaded.cfg))
     a, b = _state(model), _state(loaded)
     assert a.keys() == b.keys()
     for k in a:

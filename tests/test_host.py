@@ -152,6 +152,39 @@ def test_quantiser_entry_points_raise():
         BitshiftLinear(16, 16, 16, 5, 2, 9, 'quantlut_sym', has_kernel=True)
 
 
+def test_rope_scaling_follows_the_rotary_initialisers():
+    """rope_inv_freq against the initialisers the reference's LlamaRotaryEmbedding uses
+    (model/llama.py:39,185: transformers' ROPE_INIT_FUNCTIONS) for the static types."""
+    import torch
+    from qtip_amd.llama_decode import LlamaConfig, rope_inv_freq
+    base = dict(hidden=4096, heads=32, rope_theta=500000.0)
+    plain = rope_inv_freq(LlamaConfig(**base))
+    want = 1.0 / (500000.0**(torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    assert torch.equal(plain, want)
+    lin = rope_inv_freq(LlamaConfig(**base, rope_scaling={"type": "linear", "factor": 4.0}))
+    assert torch.allclose(lin, want / 4.0, rtol=0, atol=0)
+    l3 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+          "original_max_position_embeddings": 8192}
+    got = rope_inv_freq(LlamaConfig(**base, rope_scaling=l3))
+    # closed-form properties: short wavelengths untouched, long ones divided by the factor, monotone in between
+    wavelen = 2 * torch.pi / want
+    assert torch.equal(got[wavelen < 8192 / 4.0], want[wavelen < 8192 / 4.0])
+    assert torch.allclose(got[wavelen > 8192 / 1.0], want[wavelen > 8192 / 1.0] / 8.0)
+    mid = ~(wavelen < 8192 / 4.0) & ~(wavelen > 8192 / 1.0)
+    assert mid.any() and bool(((got[mid] <= want[mid]) & (got[mid] >= want[mid] / 8.0)).all())
+    try:
+        from transformers import LlamaConfig as HFConfig
+        from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+    except Exception:  # the library moved the table: the closed-form checks above stand alone
+        return
+    hf = HFConfig(hidden_size=4096, num_attention_heads=32, rope_theta=500000.0, rope_scaling=dict(l3),
+                  max_position_embeddings=131072)
+    ref, att = ROPE_INIT_FUNCTIONS["llama3"](hf, "cpu")
+    assert att == 1.0 and torch.allclose(got, ref, rtol=1e-6, atol=0)
+    with pytest.raises(NotImplementedError):
+        rope_inv_freq(LlamaConfig(**base, rope_scaling={"rope_type": "dynamic", "factor": 2.0}))
+
+
 def test_sampling_helpers_follow_the_generation_script():
     """top-k restriction and the exponential-race draw of eval/interactive_gen.py:15-40."""
     from qtip_amd.llama_decode import logits_to_probs, sample
