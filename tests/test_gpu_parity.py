@@ -253,6 +253,31 @@ def test_op_names_and_glue():
     assert len(cbk.kernels) >= 61
 
 
+def test_matvec_random_shapes_against_the_decoded_matrix():
+    """A seeded sweep over 40 random (m, k, bits, split) combinations - ragged k (k / 32 not a
+    multiple of 4), k ranges on both sides of the LDS staging limits, splits up to 8 - against
+    decoded weights (bit-exact against the oracle elsewhere) times x in fp64."""
+    from qtip_amd import ops
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        K = int(rng.choice([2, 3, 4]))
+        m = 32 * int(rng.integers(1, 24))
+        k = 32 * int(rng.choice([rng.integers(1, 64), rng.integers(64, 256), rng.integers(448, 900)]))
+        nwl = (k // 32 + 3) // 4
+        S = int(rng.choice([s for s in (1, 2, 4, 8) if s == 1 or nwl // s >= 16] or [1]))
+        g = torch.Generator().manual_seed(case)
+        pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+        tl = torch.randn(512, 2, generator=g).half().cuda().reshape(-1)
+        x = torch.randn(k, generator=g).half().cuda()
+        ref = ops.decode(pk, tl, m, k, K).double() @ x.double()
+        parts = ops.decompress_matvec_parts(pk, x, tl, m, k, K, nparts=S)
+        got = parts.double().sum(0).reshape(-1)
+        err = float((got - ref).abs().max() / ref.abs().max())
+        assert err <= 2e-5, (case, m, k, K, S, err)
+        full = ops.decompress_matvec(pk, x, tl, m, k, K).double().reshape(-1)
+        assert float((full - ref).abs().max() / ref.abs().max()) <= 2e-5, (case, m, k, K)
+
+
 def test_errors_raise_not_exit():
     from qtip_amd import ops
     L = make_layer(64, 64, 2)
