@@ -278,6 +278,29 @@ def test_matvec_random_shapes_against_the_decoded_matrix():
         assert float((full - ref).abs().max() / ref.abs().max()) <= 2e-5, (case, m, k, K)
 
 
+def test_gemm_random_shapes_against_the_decoded_matrix():
+    """Seeded sweep of the batched kernel: 30 random (m, k, bits, batch) combinations, batches on both
+    sides of the 16- and 32-row tile limits, against decoded weights times X in fp64 (fp32 results
+    and, rounded, the fp16 results the layer uses)."""
+    from qtip_amd import ops
+    rng = np.random.default_rng(77)
+    for case in range(30):
+        K = int(rng.choice([2, 3, 4]))
+        m = 32 * int(rng.integers(1, 40))
+        k = 32 * int(rng.choice([rng.integers(1, 64), rng.integers(64, 300), rng.integers(448, 900)]))
+        B = int(rng.choice([2, 7, 8, 15, 16, 17, 31, 32, 33, 50, 64, 70]))
+        g = torch.Generator().manual_seed(1000 + case)
+        pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+        tl = torch.randn(512, 2, generator=g).half().cuda().reshape(-1)
+        X = torch.randn(B, k, generator=g).half().cuda()
+        ref = X.double() @ ops.decode(pk, tl, m, k, K).double().T
+        got = ops.decompress_gemm(pk, X, tl, m, k, K, round_f16=False).double()
+        scale = float(ref.abs().max())
+        assert got.shape == (B, m) and float((got - ref).abs().max()) <= 2e-5 * scale, (case, m, k, K, B)
+        got16 = ops.decompress_gemm(pk, X, tl, m, k, K, round_f16=True).double()
+        assert float((got16 - ref).abs().max()) <= 1e-3 * scale, (case, m, k, K, B)
+
+
 def test_errors_raise_not_exit():
     from qtip_amd import ops
     L = make_layer(64, 64, 2)
