@@ -301,6 +301,28 @@ def test_gemm_random_shapes_against_the_decoded_matrix():
         assert float((got16 - ref).abs().max()) <= 1e-3 * scale, (case, m, k, K, B)
 
 
+@pytest.mark.parametrize("n", [2048, 4096, 8192, 11008, 12288, 5120])
+def test_hadamard_matmul_at_every_row_count_regime(n):
+    """matmul_hadU_cuda / matmul_hadUt_cuda pick their route by the number of rows (one vector,
+    a few rows, one workgroup per row, library GEMMs for the large table orders): every regime and
+    its neighbours against the fp64 Kronecker product of the table and the Sylvester matrix."""
+    import scipy.linalg
+    from qtip_amd.utils.matmul_had import get_hadK, matmul_hadU_cuda, matmul_hadUt_cuda
+    hadK, K = get_hadK(n)
+    p = n // K
+    Hp = torch.from_numpy(scipy.linalg.hadamard(p).astype(np.float64)).cuda()
+    Hk = hadK.double().cuda() if K > 1 else torch.ones(1, 1, dtype=torch.float64).cuda()
+    g = torch.Generator().manual_seed(n)
+    for rows in (1, 7, 8, 9, 40, 95, 96, 130):
+        x = torch.randn(rows, n, generator=g).cuda()
+        x3 = x.double().view(rows, K, p)
+        for fn, M in ((matmul_hadU_cuda, Hk), (matmul_hadUt_cuda, Hk.T)):
+            ref = (torch.einsum("ij,rjp->rip", M, x3) @ Hp).reshape(rows, n) * n**-0.5
+            got = fn(x, hadK.cuda() if K > 1 else None, K)
+            assert got.shape == x.shape and got.dtype == x.dtype
+            assert float((got.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max()), (n, rows, fn.__name__)
+
+
 def test_errors_raise_not_exit():
     from qtip_amd import ops
     L = make_layer(64, 64, 2)
