@@ -184,6 +184,20 @@ int qtip_rht_post_rows(void* out, int out_dtype, const void* in, int in_dtype, i
                        int order, const uint32_t* had_bits, const float* post_rows_f32, float scale,
                        void* stream);
 
+/* The output transforms of the gate and up projections and the SiLU-gated product after them, in
+ * one launch:  out = fp16(fp16(silu(gate)) * up)  (model/llama.py:399-400) with
+ * [gate | up] = fp16(post * scale * (H_order (x) H_p)(sum over in_parts of in))
+ * (lib/codebook/bitshift.py:465-472), bit-identical to qtip_rht / qtip_rht_post_rows followed by
+ * the element-wise step of qtip_rht_fused's pre_mode 2.
+ *   two_vectors == 0: one transformed vector of length n whose halves are gate and up (the fused
+ *     up/gate projection of model/llama.py:382-390); order must be even; in fp32[in_parts][n],
+ *     post fp32[n], out fp16[n / 2].
+ *   two_vectors != 0: gate and up are vectors of length n with a transform each (separate
+ *     projections); in fp32[in_parts][2][n], post fp32[2][n], out fp16[n].
+ * n / order must be a power of two >= 8; n > 4096 is what it is meant for. */
+int qtip_rht_silu_pair(void* out_f16, const float* in_f32, int in_parts, int two_vectors, int n, int order,
+                       const uint32_t* had_bits, const float* post_f32, float scale, void* stream);
+
 /* The input transforms of several QuantizedLinear layers that read the same vector, in one launch:
  * row r of out = fp16(scale * (H_order^T (x) H_p)(pre_rows[r] * rmsnorm(in))) with the RMSNorm of
  * qtip_rht_fused (model/llama.py:129-135) - q / k / v (or gate / up) of a decoder layer, each with

@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 _lib = None
 
@@ -52,6 +52,9 @@ _SIGNATURES = {
     "qtip_rht_post_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                           ctypes.c_float, ctypes.c_void_p]),
+    "qtip_rht_silu_pair": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float,
+                                          ctypes.c_void_p]),
     "qtip_rht_fused_pre_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
                                                ctypes.c_float, ctypes.c_void_p]),

@@ -1111,7 +1111,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 16; }
+int qtip_abi_version(void) { return 17; }
 
 const char* qtip_error_string(int code) {
   switch (code) {

@@ -459,6 +459,160 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   }
 }
 
+// The output transforms of gate and up and the SiLU * up that follows them, in one launch:
+//   h = fp16(fp16(silu(gate)) * up),  [gate | up] = fp16(post * scale * (H_order (x) H_p)(sum of parts))
+// (lib/codebook/bitshift.py:465-472 twice, model/llama.py:399-400).  A workgroup of the vectorised
+// form reads the whole input anyway, so it produces the gate row AND the matching up row of the
+// mix from the same loads and applies the element-wise step to the pp outputs it owns - once per
+// element, where the [SiLU * up + input transform] launch that otherwise follows repeats it in
+// every one of its workgroups.  ROWS = false: gate and up are the two halves of one transformed
+// vector (fused up/gate projection; rows iK and iK + order / 2 of the mix).  ROWS = true: two
+// vectors with a transform each (separate projections; the same row iK of either).
+template <int CH, bool ROWS>
+__global__ __launch_bounds__(kRhtThreads) void rht_vec_silu_pair_kernel(const RhtParams P) {
+  __shared__ __align__(16) float red[8192];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int A = 1 << P.logA;
+  const int iK = blockIdx.x >> P.logA, iA = blockIdx.x & (A - 1);
+  const int n = P.n, pp = P.pp, order = P.order;
+  const int iK2 = ROWS ? iK : iK + (order >> 1);
+  const float* src = reinterpret_cast<const float*>(P.in);
+  const float* src2 = ROWS ? src + P.in_row_stride : src;
+  const int OT = order << P.logA;
+  const int lcg = P.lcg;
+  const int CG = 1 << lcg;
+  const int JG = kRhtThreads >> lcg;
+  const int cg = tid & (CG - 1), jg = tid >> lcg;
+  const bool active = tid < pp;
+  const int logw = P.logw;
+  const int W = 1 << logw;
+  int cfin = tid;
+  if (W > 1) cfin = 64 * (lane & (W - 1)) + (lane >> logw) + (64 >> logw) * wave;
+  const size_t oidx1 = ((size_t)iK * A + iA) * pp + cfin;
+  const size_t oidx2 = ((size_t)iK2 * A + iA) * pp + cfin;
+  float post1 = 1.f, post2 = 1.f;
+  if (active && P.post) {
+    post1 = P.post[oidx1];
+    post2 = P.post[(ROWS ? P.post_row_stride : 0) + oidx2];
+  }
+  float z1[8], z2[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) z1[e] = z2[e] = 0.f;
+  for (int pass = 0; pass < P.npass; ++pass) {
+    const int j0 = jg + pass * JG * CH;
+    Raw8<float> xr[CH], yr[ROWS ? CH : 1];
+    uint32_t b1[CH], b2[CH];
+    bool ok[CH];
+    size_t base[CH];
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      ok[q] = j < OT;
+      base[q] = (size_t)(ok[q] ? j : 0) * pp + 8 * cg;
+      xr[q].load(src + base[q]);
+      if constexpr (ROWS) yr[q].load(src2 + base[q]);
+      b1[q] = b2[q] = 0;
+    }
+    if (order > 1) {
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        const int j = j0 + q * JG;
+        const unsigned row = (unsigned)((ok[q] ? j : 0) >> P.logA) * order;
+        const unsigned bit1 = row + iK, bit2 = row + iK2;
+        b1[q] = (P.had_bits[bit1 >> 5] >> (bit1 & 31)) & 1u;
+        b2[q] = (P.had_bits[bit2 >> 5] >> (bit2 & 31)) & 1u;
+      }
+    }
+    float v[CH][8], u[ROWS ? CH : 1][8];
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      xr[q].get(v[q]);
+      if constexpr (ROWS) yr[q].get(u[q]);
+    }
+    for (int w = 1; w < P.in_parts; ++w) {
+      Raw8<float> pr[CH], qr[ROWS ? CH : 1];
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        pr[q].load(src + w * P.part_stride + base[q]);
+        if constexpr (ROWS) qr[q].load(src2 + w * P.part_stride + base[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        float t[8];
+        pr[q].get(t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] += t[e];
+        if constexpr (ROWS) {
+          qr[q].get(t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) u[q][e] += t[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int j = j0 + q * JG;
+      if (ok[q]) {
+        const uint32_t sc = (uint32_t)__builtin_popcount(iA & (j & (A - 1))) & 1u;
+        const uint32_t s1 = (b1[q] ^ sc) << 31, s2 = (b2[q] ^ sc) << 31;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float a = v[q][e], b = ROWS ? u[q][e] : v[q][e];
+          z1[e] += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, a) ^ s1);
+          z2[e] += __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, b) ^ s2);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < 6; ++b) {
+    if (b >= lcg) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        z1[e] += lane_xor(z1[e], b);
+        z2[e] += lane_xor(z2[e], b);
+      }
+    }
+  }
+  const int NP = CG <= 64 ? 16 : JG;
+  const int part = CG <= 64 ? wave : jg;
+  const int nb0 = lcg + 3 < 6 ? lcg + 3 : 6;
+  auto finish = [&](const float z[8]) {
+    if (CG > 64 || lane < CG) {
+      float4v* dst = reinterpret_cast<float4v*>(red + part * pp + 8 * cg);
+      dst[0] = float4v{z[0], z[1], z[2], z[3]};
+      dst[1] = float4v{z[4], z[5], z[6], z[7]};
+    }
+    __syncthreads();
+    float y = 0.f;
+    if (active) {
+      for (int q = 0; q < NP; ++q) y += red[q * pp + tid];
+    }
+    __syncthreads();
+    if (active) {
+      y = wht_lanes(y, nb0, lane);
+      if (W > 1) red[tid] = y;
+    }
+    if (W > 1) {
+      __syncthreads();
+      if (active) {
+        y = red[cfin];
+        y = wht_lanes(y, logw, lane);
+      }
+    }
+    __syncthreads();  // the buffer is free for the second vector
+    return y;
+  };
+  const float y1 = finish(z1);
+  const float y2 = finish(z2);
+  if (active) {
+    const float g = (float)(_Float16)(y1 * P.scale * post1);
+    const float up = (float)(_Float16)(y2 * P.scale * post2);
+    const float sl = (float)(_Float16)(g * __builtin_amdgcn_rcpf(1.f + __expf(-g)));
+    reinterpret_cast<_Float16*>(P.out)[oidx1] = (_Float16)(sl * up);
+  }
+}
+
 template <typename TI, typename TO, bool FUSED>
 int launch_rht_vec(const RhtParams& P, dim3 grid, long loads, hipStream_t st) {
   // a prologue needs the whole row in one pass
@@ -815,6 +969,64 @@ int qtip_rht_fused(void* out, int out_dtype, const void* in, int in_dtype, int i
   P.order = order;
   P.pre_mode = pre_mode;
   return launch_rht(P, out_dtype, in_dtype, rows, stream);
+}
+
+int qtip_rht_silu_pair(void* out_f16, const float* in_f32, int in_parts, int two_vectors, int n, int order,
+                       const uint32_t* had_bits, const float* post_f32, float scale, void* stream) {
+  // n: length of one transformed vector (two_vectors: gate and up have one each; otherwise they are
+  // the halves of the one vector and out holds n / 2 values)
+  if (!out_f16 || !in_f32) return QTIP_E_NULL;
+  if (n < 1 || order < 1 || in_parts < 1 || in_parts > kMaxParts || n % order) return QTIP_E_SHAPE;
+  if (!two_vectors && (order & 1)) return QTIP_E_SHAPE;  // gate and up are whole rows of the table mix
+  const int p = n / order;
+  if (p & (p - 1)) return QTIP_E_SHAPE;
+  if (order > 1 && !had_bits) return QTIP_E_NULL;
+  int pp = p, logA = 0;
+  while (pp > kRhtThreads) {
+    pp >>= 1;
+    ++logA;
+  }
+  while (pp > 64 && ((long)order << (logA + 1)) <= 64) {
+    pp >>= 1;
+    ++logA;
+  }
+  if (pp < 8 || (reinterpret_cast<uintptr_t>(in_f32) & 15u) || ((size_t)n * 4 & 15u)) return QTIP_E_SHAPE;
+  RhtParams P{};
+  P.out = out_f16;
+  P.in = in_f32;
+  P.had_bits = had_bits;
+  P.post = post_f32;
+  P.post_row_stride = (size_t)n;
+  P.in_row_stride = (size_t)n;
+  P.part_stride = (size_t)n * (two_vectors ? 2 : 1);
+  P.scale = scale;
+  P.in_parts = in_parts;
+  P.n = n;
+  P.order = order;
+  P.logA = logA;
+  P.pp = pp;
+  int lcg = 0, logw = 0;
+  while ((8 << lcg) < pp) ++lcg;
+  while ((64 << logw) < pp) ++logw;
+  P.lcg = lcg;
+  P.logw = logw;
+  const long OT = (long)order << logA;
+  const int JGv = kRhtThreads / (pp >> 3);
+  const long loads = (OT + JGv - 1) / JGv;
+  const int ch = loads <= 1 ? 1 : loads <= 2 ? 2 : 4;
+  P.npass = (int)((loads + ch - 1) / ch);
+  const unsigned grid = (unsigned)(two_vectors ? OT : OT / 2);
+  hipStream_t st = (hipStream_t)stream;
+  if (two_vectors) {
+    if (ch == 1) rht_vec_silu_pair_kernel<1, true><<<grid, kRhtThreads, 0, st>>>(P);
+    else if (ch == 2) rht_vec_silu_pair_kernel<2, true><<<grid, kRhtThreads, 0, st>>>(P);
+    else rht_vec_silu_pair_kernel<4, true><<<grid, kRhtThreads, 0, st>>>(P);
+  } else {
+    if (ch == 1) rht_vec_silu_pair_kernel<1, false><<<grid, kRhtThreads, 0, st>>>(P);
+    else if (ch == 2) rht_vec_silu_pair_kernel<2, false><<<grid, kRhtThreads, 0, st>>>(P);
+    else rht_vec_silu_pair_kernel<4, false><<<grid, kRhtThreads, 0, st>>>(P);
+  }
+  return (int)hipGetLastError();
 }
 
 int qtip_rht_fused_pre_rows(void* out_f16, const void* in_f16, int rows, int n, int order,

@@ -199,7 +199,7 @@ class DecoderLayer(nn.Module):
         if self.fused and f['o'].can_chain_into(f['up_gate']):
             parts = f['o'].matvec_from(attn.reshape(1, -1))
             x, ug_parts = f['o'].chain_matvec(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
-            ug = f['up_gate'].transform_out(ug_parts)
+            ug = f['up_gate'].transform_out_silu(ug_parts)
         else:
             x = f['o'](attn.reshape(1, -1), residual=x)
             if self.fused:
@@ -207,11 +207,13 @@ class DecoderLayer(nn.Module):
             else:
                 ug = torch.cat([f[n](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
                                 for n in ('gate_proj', 'up_proj')], dim=-1)
+        # ug: [gate | up], or already fp16(silu(gate)) * up where the output transform paired them
+        pre = ops.PRE_SILU_MUL if ug.shape[-1] == 2 * cfg.ffn else ops.PRE_NONE
         nq = next_layer._fused_linears().get('qkv') if (next_layer is not None and next_layer.fused) else None
         if nq is not None and not f['down'].dense and f['down'].can_chain_into(nq):
-            parts = f['down'].matvec(f['down'].transform_in(ug, ops.PRE_SILU_MUL))
+            parts = f['down'].matvec(f['down'].transform_in(ug, pre))
             return f['down'].chain_matvec(parts, x, nq, next_layer.input_norm.weight, cfg.eps)
-        return f['down'](ug, ops.PRE_SILU_MUL, residual=x), None
+        return f['down'](ug, pre, residual=x), None
 
     # ---- separate projections (the layout of the published checkpoints) in grouped launches
 
@@ -276,8 +278,9 @@ class DecoderLayer(nn.Module):
         """decode_fused for separate projections with a hidden size the matvec does not transform
         itself, 12 launches: [RMSNorm + three input transforms], [q, k, v matvecs], attention with
         the three output transforms in its prologue, o as transform / matvec / transform +
-        residual, [RMSNorm + two input transforms], [gate, up matvecs], both output transforms,
-        and down as [SiLU * up + transform] / matvec / transform + residual."""
+        residual, [RMSNorm + two input transforms], [gate, up matvecs], both output transforms
+        (with SiLU * up in the same launch for vectors of up to 16384), and down as
+        [SiLU * up +] transform / matvec / transform + residual."""
         cfg = self.cfg
         f = self._fused_linears()
         qkv = [f[n] for n in ('q_proj', 'k_proj', 'v_proj')]
@@ -291,10 +294,24 @@ class DecoderLayer(nn.Module):
                                          cfg.heads, cfg.kv_heads, cfg.head_dim)
         x = f['o'](attn.reshape(1, -1), residual=x)
         gu_parts = self._group_plain(('gate_proj', 'up_proj'), x, self._su_gate_up, self.post_norm.weight)
-        g = f['gate_proj']
-        ug = ops.rht_post_rows(gu_parts.view(gu_parts.shape[0], 2, g.m), self._sv_gate_up, order=g.Kr, had_bits=g.br,
-                               scale=(g.m**-0.5) * 32.0)
-        return f['down'](ug.reshape(1, -1), ops.PRE_SILU_MUL, residual=x)
+        h, pre = self._gate_up_out(gu_parts)
+        return f['down'](h, pre, residual=x)
+
+    def _gate_up_out(self, gu_parts):
+        """(input of down, its pre_mode) from the partial sums (S, 2 * m) of the gate / up matvecs:
+        both output transforms with SiLU(gate) * up in one launch where that form exists, else
+        [gate | up] for the input transform of down to combine."""
+        g = self._fused_linears()['gate_proj']
+        parts = gu_parts.view(gu_parts.shape[0], 2, g.m)
+        scale = (g.m**-0.5) * 32.0
+        # (a workgroup of the paired form loads both vectors: past two 16-byte loads per thread and
+        # vector that costs more than the repeated SiLU it saves - 70B shapes, 28672 wide: 110.3
+        # against 111.8 tok/s; 7B shapes, 11008 wide: 484 against 468)
+        if g.m <= 16384 and ops.rht_silu_pair_ok(g.m, g.Kr, True):
+            return ops.rht_silu_pair(parts, self._sv_gate_up, order=g.Kr, had_bits=g.br,
+                                     scale=scale).reshape(1, -1), ops.PRE_NONE
+        return ops.rht_post_rows(parts, self._sv_gate_up, order=g.Kr, had_bits=g.br,
+                                 scale=scale).reshape(1, -1), ops.PRE_SILU_MUL
 
     def _group_chain(self, names, prev_parts, prev, residual, norm_weight):
         """One launch: boundary after `prev` (its output transform, residual, RMSNorm) and the
@@ -308,8 +325,9 @@ class DecoderLayer(nn.Module):
     def _decode_grouped(self, x, k_cache, v_cache, pos, inv_freq, qkv_parts, next_layer):
         """decode_fused for separate projections, 8 launches: [boundary + q, k, v matvecs] (by the
         previous layer), attention with the three output transforms in its prologue, o matvec with
-        its input transform, [boundary + gate, up matvecs], both output transforms, [SiLU * up +
-        transform], down matvec.  Returns (x, partial sums of the next layer's q, k, v)."""
+        its input transform, [boundary + gate, up matvecs], both output transforms (with SiLU * up in
+        the same launch for vectors of up to 16384), [SiLU * up +] input transform of down, down
+        matvec.  Returns (x, partial sums of the next layer's q, k, v)."""
         cfg = self.cfg
         f = self._fused_linears()
         qkv = [f[n] for n in ('q_proj', 'k_proj', 'v_proj')]
@@ -327,10 +345,8 @@ class DecoderLayer(nn.Module):
                                              cfg.heads, cfg.kv_heads, cfg.head_dim)
         po = f['o'].matvec_from(attn.reshape(1, -1))
         gu_parts, x = self._group_chain(('gate_proj', 'up_proj'), po, f['o'], x, self.post_norm.weight)
-        g = f['gate_proj']
-        ug = ops.rht_post_rows(gu_parts.view(gu_parts.shape[0], 2, g.m), self._sv_gate_up, order=g.Kr, had_bits=g.br,
-                               scale=(g.m**-0.5) * 32.0)
-        pd = f['down'].matvec(f['down'].transform_in(ug.reshape(1, -1), ops.PRE_SILU_MUL))
+        h, pre = self._gate_up_out(gu_parts)
+        pd = f['down'].matvec(f['down'].transform_in(h, pre))
         if next_layer is not None and next_layer.grouped_ok():
             parts, x = next_layer._group_chain(('q_proj', 'k_proj', 'v_proj'), pd, f['down'], x,
                                                next_layer.input_norm.weight)
@@ -391,6 +407,14 @@ class _FusedLinear:
         return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
                        post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
                        residual=residual)
+
+    def transform_out_silu(self, parts):
+        """Output transform of a fused up/gate projection; where one launch can pair the halves it
+        also applies SiLU(gate) * up and returns (1, m / 2) instead of (1, m)."""
+        if ops.rht_silu_pair_ok(self.m, self.Kr, False):
+            return ops.rht_silu_pair(parts.reshape(parts.shape[0], self.m), self.SV, order=self.Kr, had_bits=self.br,
+                                     scale=(self.m**-0.5) * 32.0).reshape(1, -1)
+        return self.transform_out(parts)
 
     def out_transform_fits_attention(self, head_dim):
         """The output transform can run in the attention kernel's prologue (head-sized slices of a

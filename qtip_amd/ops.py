@@ -392,6 +392,42 @@ def rht_post_rows(parts, post_rows, order=1, had_bits=None, scale=None, out_dtyp
     return out
 
 
+def rht_silu_pair(parts, post, order=1, had_bits=None, scale=None):
+    """fp16(fp16(silu(gate)) * up) of the transformed gate / up outputs in one launch.
+    parts (S, n) fp32 with post (n,): gate and up are the halves of one transformed vector
+    (returns (n / 2,)); parts (S, 2, n) with post (2, n): a transformed vector each (returns (n,))."""
+    require_cuda(parts, "parts", torch.float32)
+    require_cuda(post, "post", torch.float32)
+    two = parts.dim() == 3
+    if parts.dim() not in (2, 3) or post.shape != parts.shape[1:] or (two and parts.shape[1] != 2):
+        raise ValueError("parts must be (S, n) with post (n,), or (S, 2, n) with post (2, n)")
+    S, n = parts.shape[0], parts.shape[-1]
+    if order > 1:
+        require_cuda(had_bits, "had_bits", torch.int32)
+    out = torch.empty(n if two else n // 2, dtype=torch.float16, device=parts.device)
+    with torch.cuda.device(parts.device):
+        check(lib().qtip_rht_silu_pair(_ptr(out), _ptr(parts), S, int(two), n, order, _ptr(had_bits), _ptr(post),
+                                       ctypes.c_float(scale if scale is not None else n ** -0.5),
+                                       stream_ptr(parts.device)), "qtip_rht_silu_pair")
+    return out
+
+
+def rht_silu_pair_ok(n, order, two_vectors):
+    """Shapes qtip_rht_silu_pair takes (the vectorised form of the transform: rows of >= 8 values
+    per workgroup, whole rows of the table mix for either half)."""
+    p = n // order
+    if n % order or p & (p - 1) or n <= 4096 or (not two_vectors and order % 2):
+        return False
+    pp, log_a = p, 0
+    while pp > 1024:  # values per workgroup of the transform kernels
+        pp >>= 1
+        log_a += 1
+    while pp > 64 and (order << (log_a + 1)) <= 64:
+        pp >>= 1
+        log_a += 1
+    return pp >= 8
+
+
 def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head_dim):
     """Attention output (heads*head_dim,) fp16 of one new token: RoPE, cache write at `pos`
     (device int64 tensor with one element) and attention over cache slots 0..pos in one launch.

@@ -636,6 +636,59 @@ def test_output_transforms_of_several_layers_in_one_launch():
             assert torch.equal(got[r], one.reshape(-1)), (n, r)
 
 
+def test_gate_up_output_transforms_with_silu_in_one_launch():
+    """rht_silu_pair == the output transform(s) of gate and up followed by the SiLU * up prologue
+    of the next input transform: the transformed vector that the down projection reads is
+    bit-identical either way, and the paired values match fp16(silu(g)) * u computed in fp64."""
+    from qtip_amd import ops
+    from qtip_amd.utils.matmul_had import get_hadK, had_bits
+    for two, n, S in ((False, 22016, 1), (False, 57344, 2), (False, 27648, 3), (False, 106496, 1),
+                      (True, 11008, 2), (True, 28672, 1), (True, 13824, 1), (True, 8192, 2), (True, 53248, 2)):
+        g = torch.Generator().manual_seed(n + S)
+        shape = (S, 2, n) if two else (S, n)
+        parts = (torch.randn(shape, generator=g) * 0.7).cuda()
+        post = (torch.sign(torch.randn(shape[1:], generator=g) + 1e-5) * (0.5 + torch.rand(shape[1:], generator=g))).cuda()
+        hadK, order = get_hadK(n)
+        bits = had_bits(hadK, order, False, "cuda") if order > 1 else None
+        assert ops.rht_silu_pair_ok(n, order, two), (n, order, two)
+        scale = n**-0.5 * 8
+        h = ops.rht_silu_pair(parts, post, order=order, had_bits=bits, scale=scale)
+        if two:
+            gu = ops.rht_post_rows(parts, post, order=order, had_bits=bits, scale=scale).reshape(1, -1)
+        else:
+            gu = ops.rht(parts if S > 1 else parts.reshape(1, n), order=order, had_bits=bits, post=post, scale=scale,
+                         out_dtype=torch.float16, in_parts=S)
+        nh = h.numel()
+        assert gu.numel() == 2 * nh
+        gate, up = gu.reshape(-1)[:nh].double(), gu.reshape(-1)[nh:].double()
+        ref = (gate / (1 + torch.exp(-gate))).half().double() * up
+        err = (h.double() - ref).abs()
+        assert float((err / (ref.abs() + 1e-3)).max()) <= 3e-3, (two, n, S)   # 1-2 fp16 roundings
+        # what the down projection reads
+        hadL, orderL = get_hadK(nh)
+        bitsL = had_bits(hadL, orderL, True, "cuda") if orderL > 1 else None
+        su = torch.sign(torch.randn(nh, generator=g) + 1e-5).half().cuda()
+        a = ops.rht(h.reshape(1, -1), order=orderL, had_bits=bitsL, pre=su, scale=nh**-0.5, out_dtype=torch.float16)
+        b = ops.rht(gu, order=orderL, had_bits=bitsL, pre=su, scale=nh**-0.5, out_dtype=torch.float16,
+                    pre_mode=ops.PRE_SILU_MUL)
+        assert torch.equal(a.reshape(-1), b.reshape(-1)), (two, n, S)
+
+
+def test_silu_pair_rejects_what_it_does_not_cover():
+    from qtip_amd import ops
+    from qtip_amd._lib import QtipLibraryError
+    # short vectors; halves that are not whole rows of the table mix (odd order, plain power of two)
+    assert not ops.rht_silu_pair_ok(2048, 1, True)
+    assert not ops.rht_silu_pair_ok(4096 * 3, 3, False) and not ops.rht_silu_pair_ok(16384, 1, False)
+    with pytest.raises(ValueError):
+        ops.rht_silu_pair(torch.zeros(1, 3, 8192, device="cuda"), torch.ones(3, 8192, device="cuda"))
+    with pytest.raises(QtipLibraryError):
+        ops.rht_silu_pair(torch.zeros(1, 16384, device="cuda"), torch.ones(16384, device="cuda"))
+    with pytest.raises(QtipLibraryError):
+        ops.rht_silu_pair(torch.zeros(1, 3 * 4096, device="cuda"), torch.ones(3 * 4096, device="cuda"), order=3,
+                          had_bits=torch.zeros(1, dtype=torch.int32, device="cuda"))
+
+
 def test_stream_read_probe_reads_every_word_once():
     from qtip_amd import ops
     for n16 in (4, 4099, 1 << 18):
