@@ -202,7 +202,10 @@ class DecoderLayer(nn.Module):
             ug = f['up_gate'].transform_out_silu(ug_parts)
         else:
             x = f['o'](attn.reshape(1, -1), residual=x)
-            if self.fused:
+            if self.fused and not f['up_gate'].dense:
+                u = f['up_gate']
+                ug = u.transform_out_silu(u.matvec(u.transform_in(x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)))
+            elif self.fused:
                 ug = f['up_gate'](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)
             else:
                 ug = torch.cat([f[n](x, ops.PRE_RMSNORM, self.post_norm.weight, cfg.eps)

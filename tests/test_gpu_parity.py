@@ -778,6 +778,31 @@ def test_decode_of_separate_projections_with_a_table_order_hidden_size():
         assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
 
 
+@pytest.mark.parametrize("hidden,heads,ffn", [(2048, 16, 172 * 32), (2560, 20, 108 * 64)])
+def test_decode_of_separate_projections_with_paired_gate_up_transform(hidden, heads, ffn):
+    """Intermediate sizes above 4096, where the gate / up output transforms and SiLU * up are one
+    launch: the decode step (grouped launches; power-of-two and table-order hidden size) against
+    the module-by-module forward, and the same tokens with and without a HIP graph."""
+    from qtip_amd import ops
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    from qtip_amd.utils.matmul_had import get_hadK
+    assert ops.rht_silu_pair_ok(ffn, get_hadK(ffn)[1], True)
+    cfg = LlamaConfig(hidden=hidden, heads=heads, kv_heads=heads, layers=2, ffn=ffn, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64, fused=False)
+    assert all(layer.grouped_ok() or layer.grouped_plain_ok() for layer in model.layers)
+    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(2)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(5, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([5], device="cuda")
+        a = model(tok, pos)
+        b = model.decode_fused(tok, pos)
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    out, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64, fused=False), ids, 6, use_graph=True)
+    ref, _, _ = generate(LlamaDecoder(cfg, max_cache_len=64, fused=False), ids, 6, use_graph=False)
+    assert torch.equal(out, ref)
+
+
 def test_generate_falls_back_for_per_shard_transforms():
     """A model quantised with per-shard transforms (rcp != 0) is outside the fused decode step:
     generate() decodes it module by module instead of failing."""
