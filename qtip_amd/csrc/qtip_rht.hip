@@ -1013,14 +1013,14 @@ int qtip_rht_silu_pair(void* out_f16, const float* in_f32, int in_parts, int two
   const long OT = (long)order << logA;
   const int JGv = kRhtThreads / (pp >> 3);
   const long loads = (OT + JGv - 1) / JGv;
-  const int ch = loads <= 1 ? 1 : loads <= 2 ? 2 : 4;
+  // (two vectors in flight: four loads of each per pass do not fit the 128 registers of a 1024-thread workgroup)
+  const int ch = loads <= 1 ? 1 : (loads <= 2 || two_vectors) ? 2 : 4;
   P.npass = (int)((loads + ch - 1) / ch);
   const unsigned grid = (unsigned)(two_vectors ? OT : OT / 2);
   hipStream_t st = (hipStream_t)stream;
   if (two_vectors) {
     if (ch == 1) rht_vec_silu_pair_kernel<1, true><<<grid, kRhtThreads, 0, st>>>(P);
-    else if (ch == 2) rht_vec_silu_pair_kernel<2, true><<<grid, kRhtThreads, 0, st>>>(P);
-    else rht_vec_silu_pair_kernel<4, true><<<grid, kRhtThreads, 0, st>>>(P);
+    else rht_vec_silu_pair_kernel<2, true><<<grid, kRhtThreads, 0, st>>>(P);
   } else {
     if (ch == 1) rht_vec_silu_pair_kernel<1, false><<<grid, kRhtThreads, 0, st>>>(P);
     else if (ch == 2) rht_vec_silu_pair_kernel<2, false><<<grid, kRhtThreads, 0, st>>>(P);

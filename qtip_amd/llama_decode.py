@@ -282,7 +282,7 @@ class DecoderLayer(nn.Module):
         itself, 12 launches: [RMSNorm + three input transforms], [q, k, v matvecs], attention with
         the three output transforms in its prologue, o as transform / matvec / transform +
         residual, [RMSNorm + two input transforms], [gate, up matvecs], both output transforms
-        (with SiLU * up in the same launch for vectors of up to 16384), and down as
+        (with SiLU * up in the same launch for vectors above 4096), and down as
         [SiLU * up +] transform / matvec / transform + residual."""
         cfg = self.cfg
         f = self._fused_linears()
@@ -307,10 +307,7 @@ class DecoderLayer(nn.Module):
         g = self._fused_linears()['gate_proj']
         parts = gu_parts.view(gu_parts.shape[0], 2, g.m)
         scale = (g.m**-0.5) * 32.0
-        # (a workgroup of the paired form loads both vectors: past two 16-byte loads per thread and
-        # vector that costs more than the repeated SiLU it saves - 70B shapes, 28672 wide: 110.3
-        # against 111.8 tok/s; 7B shapes, 11008 wide: 484 against 468)
-        if g.m <= 16384 and ops.rht_silu_pair_ok(g.m, g.Kr, True):
+        if ops.rht_silu_pair_ok(g.m, g.Kr, True):
             return ops.rht_silu_pair(parts, self._sv_gate_up, order=g.Kr, had_bits=g.br,
                                      scale=scale).reshape(1, -1), ops.PRE_NONE
         return ops.rht_post_rows(parts, self._sv_gate_up, order=g.Kr, had_bits=g.br,
@@ -329,7 +326,7 @@ class DecoderLayer(nn.Module):
         """decode_fused for separate projections, 8 launches: [boundary + q, k, v matvecs] (by the
         previous layer), attention with the three output transforms in its prologue, o matvec with
         its input transform, [boundary + gate, up matvecs], both output transforms (with SiLU * up in
-        the same launch for vectors of up to 16384), [SiLU * up +] input transform of down, down
+        the same launch for vectors above 4096), [SiLU * up +] input transform of down, down
         matvec.  Returns (x, partial sums of the next layer's q, k, v)."""
         cfg = self.cfg
         f = self._fused_linears()
