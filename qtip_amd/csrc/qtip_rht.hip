@@ -617,11 +617,13 @@ template <typename TI, typename TO, bool FUSED>
 int launch_rht_vec(const RhtParams& P, dim3 grid, long loads, hipStream_t st) {
   // a prologue needs the whole row in one pass
   if (FUSED && P.pre_mode == PRE_RMSNORM && loads > 4) return QTIP_E_SHAPE;
-  const int ch = loads <= 1 ? 1 : loads <= 2 ? 2 : 4;
+  // (the fused form with four loads in flight spills registers: only the RMSNorm prologue, which
+  // cannot take a second pass, uses it; the sums run in the same order either way)
+  const int ch = loads <= 1 ? 1 : (loads <= 2 || (FUSED && P.pre_mode != PRE_RMSNORM)) ? 2 : 4;
   RhtParams Q = P;
   Q.npass = (int)((loads + ch - 1) / ch);
-  if (loads <= 1) rht_vec_kernel<TI, TO, 1, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
-  else if (loads <= 2) rht_vec_kernel<TI, TO, 2, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
+  if (ch == 1) rht_vec_kernel<TI, TO, 1, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
+  else if (ch == 2) rht_vec_kernel<TI, TO, 2, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
   else rht_vec_kernel<TI, TO, 4, FUSED><<<grid, kRhtThreads, 0, st>>>(Q);
   return (int)hipGetLastError();
 }
