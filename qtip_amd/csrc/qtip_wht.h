@@ -30,14 +30,28 @@ __device__ __forceinline__ float lane_xor(float v, int b) {
   return __builtin_bit_cast(float, r);
 }
 
-// Walsh-Hadamard butterflies over lane bits 0 .. nbits-1 (natural order)
+// One butterfly over lane bit b: lanes with the bit clear get v + partner, the others partner - v.
+// Written as partner + (v with its sign flipped where the bit is set): an xor and an addition (the
+// exchange rides on the addition as a DPP operand) instead of an addition, a subtraction and a
+// select; the sums are the same floating-point operations on the same operands.
+__device__ __forceinline__ float wht_stage(float v, int b, int lane) {
+  const uint32_t flip = ((uint32_t)lane << (31 - b)) & 0x80000000u;
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  if (b == 5) {
+    // the swap exchanges the upper half of its first operand with the lower half of its second:
+    // with (v, flipped v) the first result holds the lower half's values in either half and the
+    // second the upper half's, negated where they stayed at home - their sum is the butterfly
+    auto sw = __builtin_amdgcn_permlane32_swap(u, u ^ flip, false, false);
+    return __builtin_bit_cast(float, (uint32_t)sw[0]) + __builtin_bit_cast(float, (uint32_t)sw[1]);
+  }
+  return lane_xor(v, b) + __builtin_bit_cast(float, u ^ flip);
+}
+
+// Walsh-Hadamard butterflies over lane bits lo .. nbits-1 (natural order)
 __device__ __forceinline__ float wht_lanes(float v, int nbits, int lane, int lo = 0) {
 #pragma unroll
   for (int b = 0; b < 6; ++b) {
-    if (b >= lo && b < nbits) {
-      const float o = lane_xor(v, b);
-      v = ((lane >> b) & 1) ? o - v : v + o;
-    }
+    if (b >= lo && b < nbits) v = wht_stage(v, b, lane);
   }
   return v;
 }
