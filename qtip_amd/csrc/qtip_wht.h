@@ -16,10 +16,10 @@ __device__ __forceinline__ float lane_xor(float v, int b) {
   switch (b) {
     case 0: r = __builtin_amdgcn_update_dpp(0, u, 0xB1, 0xF, 0xF, false); break;  // quad_perm 1,0,3,2
     case 1: r = __builtin_amdgcn_update_dpp(0, u, 0x4E, 0xF, 0xF, false); break;  // quad_perm 2,3,0,1
-    case 2:  // xor 4 inside a row of 16: row_ror:12 brings lane+4 to the banks with bit 2 clear, row_ror:4 lane-4 to the others
-      r = __builtin_amdgcn_update_dpp(0, u, 0x12C, 0xF, 0x5, false);
-      r = __builtin_amdgcn_update_dpp(r, u, 0x124, 0xF, 0xA, false);
-      break;
+    // xor 4 and xor 16 go through the LDS crossbar: one instruction outside the vector pipe (two
+    // bank-masked row rotations do xor 4 as well, but cost two vector instructions that cannot
+    // ride on the addition; the transforms are bound by vector issue)
+    case 2: r = __builtin_amdgcn_ds_swizzle(u, 0x101F); break;                    // xor 4
     case 3: r = __builtin_amdgcn_update_dpp(0, u, 0x128, 0xF, 0xF, false); break;  // xor 8 = row_ror:8
     case 4: r = __builtin_amdgcn_ds_swizzle(u, 0x401F); break;                    // xor 16
     default: {
