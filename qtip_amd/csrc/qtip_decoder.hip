@@ -14,14 +14,20 @@ namespace {
 constexpr int kAttnThreads = 1024;
 constexpr int kMaxHeadDim = 256;
 
+// Cross-lane exchanges go through qtip_wht::lane_xor (DPP, ds_swizzle, v_permlane32_swap: a few
+// cycles each); a generic shuffle is a ds_bpermute with an LDS round trip per step, which these
+// latency-bound kernels feel.
+__device__ __forceinline__ int lane_xor_i(int v, int b) {
+  return __builtin_bit_cast(int, qtip_wht::lane_xor(__builtin_bit_cast(float, v), b));
+}
 __device__ __forceinline__ float wave_reduce_max(float v) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  for (int b = 5; b >= 0; --b) v = fmaxf(v, qtip_wht::lane_xor(v, b));
   return v;
 }
 __device__ __forceinline__ float wave_reduce_sum(float v) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  for (int b = 5; b >= 0; --b) v += qtip_wht::lane_xor(v, b);
   return v;
 }
 
@@ -256,11 +262,11 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     }
     // rows that share a wave, then one partial slice per wave
 #pragma unroll
-    for (int o = 32; o >= G; o >>= 1)
+    for (int b = 5; (1 << b) >= G; --b)
 #pragma unroll
       for (int s3 = 0; s3 < 3; ++s3)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) a[s3][e] += __shfl_xor(a[s3][e], o);
+        for (int e = 0; e < 4; ++e) a[s3][e] += qtip_wht::lane_xor(a[s3][e], b);
     if (lane < G) {
 #pragma unroll
       for (int s3 = 0; s3 < 3; ++s3)
@@ -341,9 +347,9 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
           for (int e = 0; e < 8; ++e) s += q_s[sub * dper + d8 * 8 + e] * (float)hv[e];
         }
       }
-      s += __shfl_xor(s, 1);
-      s += __shfl_xor(s, 2);
-      s += __shfl_xor(s, 4);
+      s += qtip_wht::lane_xor(s, 0);
+      s += qtip_wht::lane_xor(s, 1);
+      s += qtip_wht::lane_xor(s, 2);
       s *= sm_scale;
       if (t < nkeys) {
         if (sub == 0) p_s[t] = s;
@@ -608,9 +614,9 @@ __global__ __launch_bounds__(kHeadThreads) void greedy_pick_kernel(const _Float1
     }
   }
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const float ob = __shfl_xor(best, o);
-    const int oi = __shfl_xor(idx, o);
+  for (int b = 0; b < 6; ++b) {
+    const float ob = qtip_wht::lane_xor(best, b);
+    const int oi = lane_xor_i(idx, b);
     if (ob > best || (ob == best && oi < idx)) {
       best = ob;
       idx = oi;
@@ -706,9 +712,9 @@ __global__ __launch_bounds__(kHeadThreads) void sample_pick_kernel(const _Float1
       }
     }
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const float ob = __shfl_xor(best, o);
-      const int oi = __shfl_xor(idx, o);
+    for (int b = 0; b < 6; ++b) {
+      const float ob = qtip_wht::lane_xor(best, b);
+      const int oi = lane_xor_i(idx, b);
       if (before(ob, oi, best, idx)) {
         best = ob;
         idx = oi;
