@@ -69,7 +69,15 @@ def _qlinear(cfg, fin, fout, gen, device, K=None):
     if gen is not None:
         with torch.no_grad():
             lin.trellis.copy_(torch.randint(-32768, 32768, lin.trellis.shape, dtype=torch.int16, generator=gen))
-            lin.tlut.copy_(torch.randn(512, 2, generator=gen).half())
+            # quantlut_sym gives only the first value of a table entry a random sign
+            # (lib/codebook/bitshift.py:72-80), so the second column's mean is the mean of half the
+            # weights: a random table leaves a rank-one part mu * 1 1^T in the matrix, which the
+            # output transform collects in element 0 of every layer's output (hundreds of sigma for
+            # the widest layers; 80 layers of it overflow the fp16 residual).  Trained tables are
+            # symmetric; centre the random one.
+            tlut = torch.randn(512, 2, generator=gen)
+            tlut[:, 1] -= tlut[:, 1].mean()
+            lin.tlut.copy_(tlut.half())
             lin.SU.copy_(torch.sign(torch.randn(fin, generator=gen) + 1e-5).half())
             # decoded weights are ~N(0,1): scale so that the layer behaves like a 1/sqrt(fan_in) init
             lin.SV.copy_(torch.sign(torch.randn(fout, generator=gen) + 1e-5) / math.sqrt(fin))
