@@ -37,6 +37,12 @@ SHAPES_70B = [("qkv", 10240, 8192), ("o", 8192, 8192), ("up_gate", 57344, 8192),
 SHAPES_7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("up_gate", 22016, 4096), ("down", 4096, 11008)]
 
 
+def _distinct(toks, new):
+    """Distinct values among the `new` decoded tokens: 1 would mean a loop that decodes non-finite
+    logits (argmax of NaN is token 0 every time)."""
+    return int(toks.reshape(-1)[-new:].unique().numel())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -288,18 +294,19 @@ def main():
         from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
         model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev)
         prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
-        _, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
+        toks, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
         result["e2e_decode"] = {"model": "Llama-2-7B architecture, random init, 2-bit HYB, fused qkv and up/gate",
                                 "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1),
-                                "ms_per_token": round(1e3 / tps, 3)}
+                                "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 256)}
         del model
         torch.cuda.empty_cache()
         # the layout of the published checkpoints: seven separate projections per layer (grouped launches)
         model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev, fused=False)
-        _, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
+        toks, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
         result["e2e_decode_separate_projections"] = {
             "model": "Llama-2-7B architecture, random init, 2-bit HYB, q/k/v/o/gate/up/down separate",
-            "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1), "ms_per_token": round(1e3 / tps, 3)}
+            "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1), "ms_per_token": round(1e3 / tps, 3),
+            "distinct_new_tokens": _distinct(toks, 256)}
         del model
         torch.cuda.empty_cache()
 
@@ -310,10 +317,10 @@ def main():
         cfg70 = LlamaConfig(hidden=8192, heads=64, kv_heads=8, layers=80, ffn=28672, vocab=32000, K=2)
         model = LlamaDecoder(cfg70, max_cache_len=512, device=dev)
         prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
-        _, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
+        toks, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
         result["e2e_decode_70b"] = {"model": "Llama-2-70B architecture, random init, 2-bit HYB, fused qkv and up/gate",
                                     "prompt": 128, "new_tokens": 128, "tok_per_s": round(tps, 1),
-                                    "ms_per_token": round(1e3 / tps, 3)}
+                                    "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 128)}
         del model
         torch.cuda.empty_cache()
 
@@ -323,10 +330,10 @@ def main():
         cfg13 = LlamaConfig(hidden=5120, heads=40, kv_heads=40, layers=40, ffn=13824, vocab=32000, K=2)
         model = LlamaDecoder(cfg13, max_cache_len=512, device=dev, fused=False)
         prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
-        _, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
+        toks, dt, tps = generate(model, prompt, 128, use_graph=True, fused=True)
         result["e2e_decode_13b"] = {"model": "Llama-2-13B architecture, random init, 2-bit HYB, separate projections",
                                     "prompt": 128, "new_tokens": 128, "tok_per_s": round(tps, 1),
-                                    "ms_per_token": round(1e3 / tps, 3)}
+                                    "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 128)}
         del model
         torch.cuda.empty_cache()
 
