@@ -803,6 +803,28 @@ def test_decode_of_separate_projections_with_paired_gate_up_transform(hidden, he
     assert torch.equal(out, ref)
 
 
+def test_synthetic_model_tables_leave_no_rank_one_part():
+    """Seeded random tables have a centred second column (only the first value of an entry gets
+    the hash's sign, lib/codebook/bitshift.py:72-80): without that every matrix carries mu * 1 1^T
+    and element 0 of each layer's output grows by hundreds of sigma.  The widest output of a
+    random layer stays within a few sigma and a deep random model decodes finite logits."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder
+    cfg = LlamaConfig(hidden=2048, heads=16, kv_heads=4, layers=40, ffn=172 * 32, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=32)
+    for layer in model.layers:
+        for lin in layer._fused_linears().values():
+            assert abs(float(lin.lin.tlut[:, 1].float().mean())) < 2e-3
+    x = torch.randn(4, cfg.ffn, generator=torch.Generator().manual_seed(0)).half().cuda()
+    y = model.layers[0].down(x).float()
+    assert float(y.abs().max()) < 8 * float(y.std())
+    ids = torch.randint(0, cfg.vocab, (1, 12), generator=torch.Generator().manual_seed(3)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(12, device="cuda"))
+        st = model.decode_fused(lg[:, -1].argmax(-1, keepdim=True), torch.tensor([12], device="cuda"))
+    assert bool(torch.isfinite(lg).all()) and bool(torch.isfinite(st).all())
+    assert float(lg.float().abs().max()) < 100
+
+
 def test_generate_falls_back_for_per_shard_transforms():
     """A model quantised with per-shard transforms (rcp != 0) is outside the fused decode step:
     generate() decodes it module by module instead of failing."""
