@@ -470,7 +470,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
 // vectors with a transform each (separate projections; the same row iK of either).
 template <int CH, bool ROWS>
 __global__ __launch_bounds__(kRhtThreads) void rht_vec_silu_pair_kernel(const RhtParams P) {
-  __shared__ __align__(16) float red[8192];
+  __shared__ __align__(16) float red[2 * 8192];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int A = 1 << P.logA;
   const int iK = blockIdx.x >> P.logA, iA = blockIdx.x & (A - 1);
@@ -577,34 +577,42 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_silu_pair_kernel(const Rh
   const int NP = CG <= 64 ? 16 : JG;
   const int part = CG <= 64 ? wave : jg;
   const int nb0 = lcg + 3 < 6 ? lcg + 3 : 6;
-  auto finish = [&](const float z[8]) {
-    if (CG > 64 || lane < CG) {
-      float4v* dst = reinterpret_cast<float4v*>(red + part * pp + 8 * cg);
-      dst[0] = float4v{z[0], z[1], z[2], z[3]};
-      dst[1] = float4v{z[4], z[5], z[6], z[7]};
+  // both vectors go through the reduction and the pp-point transform side by side: three
+  // barriers for the pair
+  float* red1 = red;
+  float* red2 = red + 8192;
+  if (CG > 64 || lane < CG) {
+    float4v* d1 = reinterpret_cast<float4v*>(red1 + part * pp + 8 * cg);
+    float4v* d2 = reinterpret_cast<float4v*>(red2 + part * pp + 8 * cg);
+    d1[0] = float4v{z1[0], z1[1], z1[2], z1[3]};
+    d1[1] = float4v{z1[4], z1[5], z1[6], z1[7]};
+    d2[0] = float4v{z2[0], z2[1], z2[2], z2[3]};
+    d2[1] = float4v{z2[4], z2[5], z2[6], z2[7]};
+  }
+  __syncthreads();
+  float y1 = 0.f, y2 = 0.f;
+  if (active) {
+    for (int q = 0; q < NP; ++q) {
+      y1 += red1[q * pp + tid];
+      y2 += red2[q * pp + tid];
     }
-    __syncthreads();
-    float y = 0.f;
-    if (active) {
-      for (int q = 0; q < NP; ++q) y += red[q * pp + tid];
-    }
-    __syncthreads();
-    if (active) {
-      y = wht_lanes(y, nb0, lane);
-      if (W > 1) red[tid] = y;
-    }
+  }
+  if (W > 1) __syncthreads();  // the partial vectors are consumed before the buffers are reused
+  if (active) {
+    y1 = wht_lanes(y1, nb0, lane);
+    y2 = wht_lanes(y2, nb0, lane);
     if (W > 1) {
-      __syncthreads();
-      if (active) {
-        y = red[cfin];
-        y = wht_lanes(y, logw, lane);
-      }
+      red1[tid] = y1;
+      red2[tid] = y2;
     }
-    __syncthreads();  // the buffer is free for the second vector
-    return y;
-  };
-  const float y1 = finish(z1);
-  const float y2 = finish(z2);
+  }
+  if (W > 1) {
+    __syncthreads();
+    if (active) {
+      y1 = wht_lanes(red1[cfin], logw, lane);
+      y2 = wht_lanes(red2[cfin], logw, lane);
+    }
+  }
   if (active) {
     const float g = (float)(_Float16)(y1 * P.scale * post1);
     const float up = (float)(_Float16)(y2 * P.scale * post2);
