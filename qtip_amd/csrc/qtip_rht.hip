@@ -192,10 +192,10 @@ __global__ __launch_bounds__(kRhtThreads) void rht_kernel(const RhtParams P) {
       y = z[0];  // JG == 1 implies pp == 1024 and RI == 1
     }
   }
-  if (JG > 1) __syncthreads();
   // ---- pp-point transform
   const int logw = P.logw;
   const int W = 1 << logw;  // waves holding one row
+  if (JG > 1 && W > 1) __syncthreads();  // the buffer is reused only when a row spans several waves
   const int nb0 = logc < 6 ? logc : 6;
   int cfin = col;
   if (active) {
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(kRhtThreads) void rht_vec_kernel(const RhtParams P)
   if (active) {
     for (int q = 0; q < NP; ++q) y += red[q * pp + tid];
   }
-  __syncthreads();
+  if (W > 1) __syncthreads();  // the buffer is reused only when a row spans several waves
   // ---- pp-point transform of column tid
   const int nb0 = lcg + 3 < 6 ? lcg + 3 : 6;  // log2(pp), at most the six lane bits
   if (active) {
