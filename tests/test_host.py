@@ -209,3 +209,16 @@ def test_sampling_helpers_follow_the_generation_script():
     tok, _ = sample(lg)
     freq = torch.bincount(tok.flatten(), minlength=3).float() / 6000
     assert (freq - torch.tensor([0.7, 0.2, 0.1])).abs().max() < 0.03
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus value ends with a message and a non-zero
+    status before the library or a device is touched."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
