@@ -6,8 +6,12 @@
  *   - all pointers are DEVICE pointers on the current HIP device, plain C types;
  *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
  *   - asynchronous: the call enqueues work and returns; it never synchronises,
- *     allocates, frees or queries device properties, so it may be recorded
- *     into a HIP graph;
+ *     allocates or frees, so it may be recorded into a HIP graph.  The first
+ *     launcher call on a device runs that device's one-time set-up
+ *     (qtip_init: CU count, LDS opt-in per kernel) if qtip_init has not been
+ *     called there - unless its stream is being captured: then nothing is
+ *     recorded and the call returns QTIP_E_NOT_INIT, so a caller whose first
+ *     call would be inside a stream capture calls qtip_init() beforehand;
  *   - returns 0 on success, a negative QTIP_E_* code for rejected arguments
  *     (nothing was launched), or a positive hipError_t from the launch.  It
  *     never terminates the process (the reference's launcher exits on error,
@@ -34,12 +38,20 @@ extern "C" {
 #define QTIP_E_ALIGN (-3)     /* a pointer is not 16-byte aligned */
 #define QTIP_E_WORKSPACE (-4) /* workspace smaller than qtip_matvec_workspace_bytes */
 #define QTIP_E_DTYPE (-5)     /* unknown dtype code */
+#define QTIP_E_NOT_INIT (-7)  /* first call on this device came inside a stream capture */
 
 #define QTIP_F16 0
 #define QTIP_F32 1
 
 /* Library ABI version (bumped when a signature changes). */
 int qtip_abi_version(void);
+
+/* One-time set-up for the CURRENT device: reads the CU count, opts every kernel into its LDS
+ * size.  Allocates nothing and does not synchronise.  Idempotent and thread-safe; returns 0 or a hipError_t.  Every launcher
+ * runs it on first use of a device, so calling it is only required before a stream capture
+ * whose first recorded call would otherwise be the library's first call on that device.
+ * No counterpart in the reference (its templates need no run-time set-up). */
+int qtip_init(void);
 
 /* Text for a return code of any launcher below (static storage). */
 const char* qtip_error_string(int code);

@@ -59,6 +59,8 @@ static inline void lookup(const uint16_t* tlut, uint32_t s, uint16_t w[2]) {
 int qtip_oracle_decode(const uint8_t* packed, const uint16_t* tlut, int m, int k, int K,
                        uint16_t* out) {
   if (m % 32 || k % 32 || K < 2 || K > 4) return -1;
+  /* 32-row blocks are independent of each other (OpenMP only spreads them over the host cores) */
+#pragma omp parallel for schedule(static)
   for (int i0 = 0; i0 < m / 32; ++i0)
     for (int i1 = 0; i1 < k / 32; ++i1) {
       const uint8_t* blk = packed + ((size_t)i0 * (k / 32) + i1) * 128 * K;
@@ -82,6 +84,8 @@ int qtip_oracle_matvec(const uint8_t* packed, const uint16_t* tlut, const uint16
                        int K, double* out) {
   if (m % 32 || k % 32 || K < 2 || K > 4) return -1;
   for (int i = 0; i < m; ++i) out[i] = 0.0;
+  /* a row block owns its 32 outputs; the sum over a row keeps its serial order */
+#pragma omp parallel for schedule(static)
   for (int i0 = 0; i0 < m / 32; ++i0)
     for (int i1 = 0; i1 < k / 32; ++i1) {
       const uint8_t* blk = packed + ((size_t)i0 * (k / 32) + i1) * 128 * K;

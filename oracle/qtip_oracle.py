@@ -346,7 +346,7 @@ def hadamard_transform(x: np.ndarray, transpose: bool = False) -> np.ndarray:
 # ----------------------------------------------------------------------------
 
 
-def bitshift_linear_forward(inp, packed, SU, SV, tlut, K, return_parts=False):
+def bitshift_linear_forward(inp, packed, SU, SV, tlut, K, return_parts=False, matvec_fn=None):
     """Restates BitshiftLinear.forward, eval mode, rcp=0
     (lib/codebook/bitshift.py:415-472) with its cast points:
 
@@ -358,6 +358,10 @@ def bitshift_linear_forward(inp, packed, SU, SV, tlut, K, return_parts=False):
     so the result is the value the device's fp32 pipeline approximates.  For
     more than one row the reference rounds y0 to fp16 once (:489); that
     rounding is applied here as well.
+
+    matvec_fn(x4_row) -> (m,) float64, if given, supplies hatW x4 row by row
+    (the C restatement for the full-size matrices, where a dense float64 copy
+    of hatW would not fit in memory).
     """
     SU = np.asarray(SU)
     SV = np.asarray(SV)
@@ -366,8 +370,11 @@ def bitshift_linear_forward(inp, packed, SU, SV, tlut, K, return_parts=False):
     x1 = x0.astype(np.float32) * SU.astype(np.float32)
     x2 = hadamard_transform(x1, transpose=True)
     x4 = (x2 / 32.0).astype(np.float32).astype(np.float16)
-    w = decode_kernel(packed, tlut, m, n, K).astype(np.float64)
-    y0 = x4.astype(np.float64) @ w.T
+    if matvec_fn is not None:
+        y0 = np.stack([np.asarray(matvec_fn(row), dtype=np.float64) for row in x4])
+    else:
+        w = decode_kernel(packed, tlut, m, n, K).astype(np.float64)
+        y0 = x4.astype(np.float64) @ w.T
     if x0.shape[0] > 1:
         y0 = y0.astype(np.float16).astype(np.float64)
     y1 = hadamard_transform(y0, transpose=False)

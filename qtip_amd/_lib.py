@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _lib = None
 
@@ -24,6 +24,7 @@ class QtipLibraryError(RuntimeError):
 
 _SIGNATURES = {
     "qtip_abi_version": (ctypes.c_int, []),
+    "qtip_init": (ctypes.c_int, []),
     "qtip_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "qtip_decode": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p]),
     "qtip_matvec_split": (ctypes.c_int, [ctypes.c_int] * 3),
@@ -108,6 +109,21 @@ def lib():
     return _lib
 
 
+_INITIALISED = set()
+
+
+def init_device(device=None):
+    """qtip_init() for `device` (default: the current one), once per device and process: the
+    library's one-time set-up, kept out of any later stream capture."""
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index
+    if dev is None:
+        dev = torch.cuda.current_device()
+    if dev not in _INITIALISED:
+        with torch.cuda.device(dev):
+            check(lib().qtip_init(), "qtip_init")
+        _INITIALISED.add(dev)
+
+
 def check(code, what):
     if code != 0:
         msg = lib().qtip_error_string(code).decode()
@@ -115,6 +131,9 @@ def check(code, what):
 
 
 def stream_ptr(device):
+    """Current stream of `device` as the launchers take it; also the point where a device the
+    library has not met yet gets its one-time set-up (every launch passes through here)."""
+    init_device(device)
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/qtip_hip.h"
 #include "qtip_device.h"
 #include "qtip_wht.h"
@@ -219,11 +221,11 @@ __device__ __forceinline__ void load_x_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t
 // xs[e] = fp16(scale * (H_k (su * x))[e]) for the whole vector, written to LDS where the
 // kernel keeps its activations.  Every workgroup computes the whole transform (a few thousand
 // butterflies per thread, hidden behind the latency of the first weight loads) - it replaces
-// a separate transform launch.  `scratch` (k + k/64 floats) is the table's LDS, not yet built.
+// a separate transform launch.  `xchg` (k + k/64 floats) is the table's LDS, not yet built.
 // Element e = [wave 4][lane 6][i]: butterflies over the register bits, the six lane bits and,
 // after one exchange through LDS that swaps the wave bits with the low four lane bits, the rest.
 template <int EPT>
-__device__ __forceinline__ void xform_prologue(const float v_in[8], float scale, float* scratch,
+__device__ __forceinline__ void xform_prologue(const float v_in[8], float scale, float* xchg,
                                                _Float16* xs, int tid, int lane, int wave) {
   using namespace qtip_wht;
   float v[EPT];
@@ -235,13 +237,13 @@ __device__ __forceinline__ void xform_prologue(const float v_in[8], float scale,
 #pragma unroll
   for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(v[i], 6, lane);
 #pragma unroll
-  for (int i = 0; i < EPT; ++i) scratch[xidx<EPT>(e_nat + i)] = v[i];
+  for (int i = 0; i < EPT; ++i) xchg[xidx<EPT>(e_nat + i)] = v[i];
   __syncthreads();
   _Float16 o[EPT];
 #pragma unroll
-  for (int i = 0; i < EPT; ++i) o[i] = (_Float16)(wht_lanes(scratch[xidx<EPT>(e_swp + i)], 4, lane) * scale);
+  for (int i = 0; i < EPT; ++i) o[i] = (_Float16)(wht_lanes(xchg[xidx<EPT>(e_swp + i)], 4, lane) * scale);
   st_f16<EPT>(xs + e_swp, o);
-  __syncthreads();  // scratch is free for the table, xs is complete
+  __syncthreads();  // xchg is free for the table, xs is complete
 }
 
 // XFORM == 2: the whole boundary between two linear layers of a decoder in front of the matvec,
@@ -558,12 +560,12 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       default: chain_compute<8>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
     }
   } else if constexpr (XFORM == 1) {
-    float* scratch = reinterpret_cast<float*>(smem);
+    float* xchg = reinterpret_cast<float*>(smem);
     _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
     switch (k >> 10) {
-      case 2: xform_prologue<2>(xraw, xscale, scratch, xs, tid, lane, wave); break;
-      case 4: xform_prologue<4>(xraw, xscale, scratch, xs, tid, lane, wave); break;
-      default: xform_prologue<8>(xraw, xscale, scratch, xs, tid, lane, wave); break;
+      case 2: xform_prologue<2>(xraw, xscale, xchg, xs, tid, lane, wave); break;
+      case 4: xform_prologue<4>(xraw, xscale, xchg, xs, tid, lane, wave); break;
+      default: xform_prologue<8>(xraw, xscale, xchg, xs, tid, lane, wave); break;
     }
   }
 #pragma unroll
@@ -995,74 +997,116 @@ __global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict_
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-struct DeviceInfo {
-  int cus = 0;
-  bool ok = false;
-};
-
-// One-time per-process set-up (CU count, LDS opt-in).  Runs on the first call
-// of any launcher; callers that record HIP graphs make one eager call first.
-DeviceInfo& device_info() {
-  static DeviceInfo info = [] {
-    DeviceInfo d;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return d;
-    int cus = 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-      return d;
-    d.cus = cus > 0 ? cus : 256;
-    d.ok = true;
-    return d;
-  }();
-  return info;
-}
-
 template <typename F>
 hipError_t allow_lds(F* fn, size_t bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-
-hipError_t setup_once() {
-  static hipError_t status = [] {
-    hipError_t e;
+hipError_t allow_lds_all() {
+  hipError_t e;
 #define QTIP_ALLOW(fn, bytes) \
   if ((e = allow_lds(fn, bytes)) != hipSuccess) return e;
-    QTIP_ALLOW((decode_kernel<2>), kDecodeLds)
-    QTIP_ALLOW((decode_kernel<3>), kDecodeLds)
-    QTIP_ALLOW((decode_kernel<4>), kDecodeLds)
-    QTIP_ALLOW((matvec_kernel<2, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<3, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
-    QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, 1>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, 1>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, 1>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<2, 2, true, 2>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<3, 2, true, 2>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((matvec_kernel<4, 2, true, 2>), kMatvecLds + kMatvecXBytes)
-    QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
-    QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
+  QTIP_ALLOW((decode_kernel<2>), kDecodeLds)
+  QTIP_ALLOW((decode_kernel<3>), kDecodeLds)
+  QTIP_ALLOW((decode_kernel<4>), kDecodeLds)
+  QTIP_ALLOW((matvec_kernel<2, 2, false>), kMatvecLds)
+  QTIP_ALLOW((matvec_kernel<3, 2, false>), kMatvecLds)
+  QTIP_ALLOW((matvec_kernel<4, 2, false>), kMatvecLds)
+  QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true, 2, false, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true, 0, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true, 1>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 2>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<3, 2, true, 2>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<4, 2, true, 2>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((gemm_kernel<2, 1, 4, 16>), kGemmLds)
+  QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
+  QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
+  QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
+  QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
+  QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
 #undef QTIP_ALLOW
-    return hipSuccess;
-  }();
-  return status;
+  return hipSuccess;
+}
+
+// Per-device set-up: CU count and LDS opt-in of every kernel.  qtip_init() runs it for the current device; a launcher that meets a device for the
+// first time runs it too (none of it allocates or synchronises, but hipFuncSetAttribute is not
+// a call to make while a stream is being captured: callers that record graphs call qtip_init()
+// first).
+struct DeviceState {
+  int cus = 0;
+  hipError_t status = hipErrorNotInitialized;
+  bool done = false;
+  bool refused = false;  // first use of the device inside a stream capture: set-up not run
+};
+constexpr int kMaxDevices = 64;
+DeviceState g_devices[kMaxDevices];
+std::mutex g_devices_mutex;
+
+// A launcher that meets a device for the first time while its stream is being captured does
+// not run the set-up (hipFuncSetAttribute and friends are no calls to make inside a capture):
+// it reports QTIP_E_NOT_INIT (`refused` in the state it gets back).
+
+// State of the current device, set up on first use; status != hipSuccess if that failed.
+// `launching`: the caller is about to enqueue work on `st`.
+DeviceState& device_state(bool launching = false, hipStream_t st = nullptr) {
+  static thread_local DeviceState none;  // no usable device / refused: status is an error
+  int dev = -1;
+  const hipError_t ge = hipGetDevice(&dev);
+  if (ge != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    none.status = ge != hipSuccess ? ge : hipErrorInvalidDevice;
+    none.refused = false;
+    return none;
+  }
+  std::lock_guard<std::mutex> lock(g_devices_mutex);
+  DeviceState& d = g_devices[dev];
+  if (d.done) return d;
+  if (launching) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    const hipError_t ce = hipStreamIsCapturing(st, &cs);
+    if (ce == hipErrorStreamCaptureImplicit || (ce == hipSuccess && cs != hipStreamCaptureStatusNone)) {
+      none.status = hipErrorNotInitialized;
+      none.refused = true;
+      return none;
+    }
+    if (ce != hipSuccess) (void)hipGetLastError();  // the query's own error is not the caller's
+  }
+  int cus = 0;
+  hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess) e = allow_lds_all();
+  d.status = e;
+  if (e == hipSuccess) {
+    d.cus = cus > 0 ? cus : 256;
+    d.done = true;  // a failed set-up is tried again by the next call
+  }
+  return d;
+}
+
+// the launchers below read the CU count through this view
+struct DeviceInfo {
+  int cus;
+  bool ok;
+};
+DeviceInfo device_info() {
+  const DeviceState& d = device_state();
+  return DeviceInfo{d.cus, d.status == hipSuccess};
+}
+// return code of a launcher for the state of its device: 0, QTIP_E_NOT_INIT or a hipError_t
+int ready_code(void* stream) {
+  const DeviceState& d = device_state(true, (hipStream_t)stream);
+  return d.refused ? QTIP_E_NOT_INIT : (int)d.status;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1111,7 +1155,9 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 17; }
+int qtip_abi_version(void) { return 18; }
+
+int qtip_init(void) { return (int)device_state().status; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -1121,6 +1167,9 @@ const char* qtip_error_string(int code) {
     case QTIP_E_ALIGN: return "qtip: pointer not 16-byte aligned";
     case QTIP_E_WORKSPACE: return "qtip: workspace too small";
     case QTIP_E_DTYPE: return "qtip: unknown dtype code";
+    case QTIP_E_NOT_INIT:
+      return "qtip: first call on this device came inside a stream capture; call qtip_init() (or any "
+             "launcher) on the device before capturing";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "qtip: unknown error";
   }
 }
@@ -1131,10 +1180,8 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
   if (rc) return rc;
   if (!aligned16(out_f16) || !aligned16(packed) || (reinterpret_cast<uintptr_t>(tlut) & 3u))
     return QTIP_E_ALIGN;
-  DeviceInfo& di = device_info();
-  if (!di.ok) return (int)hipErrorInvalidDevice;
-  hipError_t e = setup_once();
-  if (e != hipSuccess) return (int)e;
+  if ((rc = ready_code(stream))) return rc;
+  const DeviceInfo di = device_info();
   const long total = (long)(m >> 5) * (((k >> 5) + 3) >> 2);
   long want = (total + kWaves - 1) / kWaves;
   const int grid = (int)(want < di.cus ? want : di.cus);
@@ -1152,14 +1199,14 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
 
 int qtip_matvec_split(int m, int k, int bits) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
-  DeviceInfo& di = device_info();
+  const DeviceInfo di = device_info();
   if (!di.ok) return 0;
   return choose_split(m, k, bits, di.cus, false);
 }
 
 size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
-  DeviceInfo& di = device_info();
+  const DeviceInfo di = device_info();
   if (!di.ok) return 0;
   const int S = choose_split(m, k, bits, di.cus, true);
   return S > 1 ? (size_t)S * m * sizeof(float) : 0;
@@ -1168,7 +1215,7 @@ size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
 static int launch_matvec(float* dst, const void* packed, const void* x_f16, const void* tlut, int m,
                          int k, int bits, int S, hipStream_t st, const void* su_f16 = nullptr,
                          float xscale = 1.f, const ChainArgs* chain = nullptr) {
-  DeviceInfo& di = device_info();
+  const DeviceInfo di = device_info();
   const long units = (long)(m >> 5) * S;
   long grid = units < di.cus ? units : di.cus;
   grid -= grid % S;  // a workgroup keeps one k range (units is a multiple of S, so grid >= S)
@@ -1226,21 +1273,19 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
 }
 
 static int check_matvec(const void* out, const void* packed, const void* x_f16, const void* tlut,
-                        int m, int k, int bits) {
+                        int m, int k, int bits, void* stream) {
   int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (!aligned16(packed) || (reinterpret_cast<uintptr_t>(x_f16) & 7u) ||
       (reinterpret_cast<uintptr_t>(tlut) & 3u) || (reinterpret_cast<uintptr_t>(out) & 3u))
     return QTIP_E_ALIGN;
-  if (!device_info().ok) return (int)hipErrorInvalidDevice;
-  hipError_t e = setup_once();
-  return e == hipSuccess ? QTIP_OK : (int)e;
+  return ready_code(stream);
 }
 
 int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x_f16,
                                  const void* tlut, int m, int k, int bits, int nparts,
                                  void* stream) {
-  int rc = check_matvec(parts, packed, x_f16, tlut, m, k, bits);
+  int rc = check_matvec(parts, packed, x_f16, tlut, m, k, bits, stream);
   if (rc) return rc;
   if (nparts < 1 || nparts > kMaxSplit || nparts > ((((k >> 5) + 3) >> 2))) return QTIP_E_SHAPE;
   return launch_matvec(parts, packed, x_f16, tlut, m, k, bits, nparts, (hipStream_t)stream);
@@ -1249,7 +1294,7 @@ int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x
 int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const void* x_raw_f16,
                                      const void* su_f16, float scale, const void* tlut, int m, int k,
                                      int bits, int nparts, void* stream) {
-  int rc = check_matvec(parts, packed, x_raw_f16, tlut, m, k, bits);
+  int rc = check_matvec(parts, packed, x_raw_f16, tlut, m, k, bits, stream);
   if (rc) return rc;
   if (!su_f16) return QTIP_E_NULL;
   if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
@@ -1264,7 +1309,7 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
                                        const void* residual_f16, const void* norm_w_f16, float eps,
                                        const void* su_f16, float scale_in, void* x_out_f16,
                                        void* stream) {
-  int rc = check_matvec(parts, packed, su_f16, tlut, m, k, bits);
+  int rc = check_matvec(parts, packed, su_f16, tlut, m, k, bits, stream);
   if (rc) return rc;
   if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
   if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
@@ -1369,7 +1414,7 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
   if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
   long m_total = 0;
   for (int g = 0; g < ngroups; ++g) {
-    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits);
+    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits, stream);
     if (rc) return rc;
     if (!aligned16(su_f16[g])) return QTIP_E_ALIGN;
     m_total += m[g];
@@ -1417,7 +1462,7 @@ int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* p
   if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
   long m_total = 0;
   for (int g = 0; g < ngroups; ++g) {
-    int rc = check_matvec(parts, packed[g], x_f16[g], tlut[g], m[g], k, bits);
+    int rc = check_matvec(parts, packed[g], x_f16[g], tlut[g], m[g], k, bits, stream);
     if (rc) return rc;
     if (!aligned16(x_f16[g])) return QTIP_E_ALIGN;
     m_total += m[g];
@@ -1446,7 +1491,7 @@ int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* p
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,
                            int m, int k, int bits, void* workspace, size_t workspace_bytes,
                            void* stream) {
-  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits);
+  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits, stream);
   if (rc) return rc;
   int S = 1;
   if (workspace) {
@@ -1474,7 +1519,7 @@ static int gemm_split(int m, int k, int cus) {
 
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4 || batch < 1) return 0;
-  DeviceInfo& di = device_info();
+  const DeviceInfo di = device_info();
   if (!di.ok) return 0;
   const int S = gemm_split(m, k, di.cus);
   return S > 1 ? (size_t)S * (batch < 32 ? batch : 32) * m * sizeof(float) : 0;
@@ -1489,10 +1534,8 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   if (!aligned16(packed) || !aligned16(x_f16) || (reinterpret_cast<uintptr_t>(tlut) & 3u) ||
       (reinterpret_cast<uintptr_t>(out) & 3u))
     return QTIP_E_ALIGN;
-  DeviceInfo& di = device_info();
-  if (!di.ok) return (int)hipErrorInvalidDevice;
-  hipError_t e = setup_once();
-  if (e != hipSuccess) return (int)e;
+  if ((rc = ready_code(stream))) return rc;
+  const DeviceInfo di = device_info();
   int S = 1;
   if (workspace) {
     S = gemm_split(m, k, di.cus);

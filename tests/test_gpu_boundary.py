@@ -1,0 +1,56 @@
+"""GPU: behaviour of the C ABI at its edges - set-up, stream capture, more than one stream."""
+import os
+import subprocess
+import sys
+import textwrap
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_first_call_inside_a_capture_is_a_defined_error_then_init_and_capture_work():
+    """A process whose very first library call is a launcher on a capturing stream: the launcher
+    records nothing and returns QTIP_E_NOT_INIT; after qtip_init() the same capture records, and
+    its replays equal the eager result.  (Own process: set-up happens once per process.)"""
+    code = textwrap.dedent("""
+        import ctypes, sys
+        import torch
+        sys.path.insert(0, %r)
+        from qtip_amd._lib import LIB_PATH
+        lb = ctypes.CDLL(LIB_PATH)
+        lb.qtip_decompress_matvec.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        m, k, K = 512, 2048, 2
+        g = torch.Generator().manual_seed(0)
+        pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+        tl = torch.randn(512, 2, generator=g).half().cuda()
+        x = torch.randn(k, generator=g).half().cuda()
+        out = torch.zeros(m, device="cuda")
+        def launch():
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            return lb.qtip_decompress_matvec(out.data_ptr(), pk.data_ptr(), x.data_ptr(), tl.data_ptr(), m, k, K, None, 0, st)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rc_first = launch()
+            y = x * 2  # the refused call recorded nothing; keep the capture non-empty
+        assert rc_first == -7, rc_first
+        assert lb.qtip_init() == 0
+        assert launch() == 0
+        torch.cuda.synchronize()
+        eager = out.clone()
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2):
+            assert launch() == 0
+        for _ in range(3):
+            out.zero_()
+            graph2.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+        assert float(eager.abs().max()) > 0
+        print("ok")
+    """) % ROOT
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and "ok" in res.stdout, res.stdout + res.stderr

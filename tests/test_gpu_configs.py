@@ -1,0 +1,129 @@
+"""GPU: the benchmark configurations at their full size against the CPU oracle.
+
+Every matrix shape of the Llama-2-7B set (2, 3 and 4 bits), of the Llama-2-70B set (2 bits) and
+of the 4-bit batched product runs here at its real size, the sizes the reference's own
+functional test uses (qtip-kernels/test_decompress_matvec.py:9-38, 275-301): these are the
+shapes with several work units per workgroup, uneven unit counts (320 or 1792 row blocks on
+256 workgroups) and activations staged in two halves, which reduced shapes do not reach.
+Decoded weights are compared bit for bit with the C restatement of the decode; matvec, layer
+and batched outputs within max-rel 1e-2 / mean-rel 1e-3 of a float64 evaluation on the
+bit-exact weights (relative to the largest / mean magnitude of the oracle's output).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import qtip_oracle as O
+from synth import make_layer
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL = 1e-2
+MEAN_REL = 1e-3
+
+SET_7B = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]
+SET_70B = [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]
+MATVEC_CASES = [(m, k, K) for K in (2, 3, 4) for (m, k) in SET_7B] + [(m, k, 2) for (m, k) in SET_70B]
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_errors(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    d = np.abs(got - ref)
+    return d.max() / np.abs(ref).max(), d.mean() / np.abs(ref).mean()
+
+
+def assert_close(got, ref, max_rel=MAX_REL, mean_rel=MEAN_REL):
+    mx, mn = rel_errors(got, ref)
+    assert mx <= max_rel and mn <= mean_rel, (mx, mn)
+
+
+@pytest.mark.parametrize("m,k,K", MATVEC_CASES)
+def test_matrix_at_full_size(m, k, K):
+    """decode bit-exact; matvec with and without the k split, as partial vectors, through the
+    registered op and through BitshiftLinear.forward, all against the oracle."""
+    import qtip_amd.codebook  # noqa: F401  (registers the quip_lib ops)
+    from qtip_amd import ops
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from qtip_amd.utils import matmul_had as mh
+    L = make_layer(m, k, K, seed=7 * m + k + K)
+    pk, tl = dev(L["packed"]), dev(L["tlut"])
+    x = L["x"].reshape(-1)
+
+    got_w = ops.decode(pk, tl, m, k, K).cpu().numpy()
+    ref_w = c_oracle.decode(L["packed"], L["tlut"], m, k, K)
+    assert np.array_equal(got_w.view(np.uint16), ref_w.view(np.uint16))
+    del got_w, ref_w
+
+    ref = c_oracle.matvec(L["packed"], x, L["tlut"], m, k, K)
+    for split in (True, False):
+        got = ops.decompress_matvec(pk, dev(x), tl, m, k, K, split_k=split).cpu().numpy()
+        assert_close(got, ref)
+    parts = ops.decompress_matvec_parts(pk, dev(x), tl, m, k, K)
+    assert_close(parts.double().sum(0).cpu().numpy(), ref)
+    op = getattr(torch.ops.quip_lib, f"decompress_matvec_qtip_{m}_1_{k}_{K}")
+    assert_close(op(pk, dev(L["x"]).float(), tl).cpu().numpy().reshape(-1), ref)
+
+    layer = BitshiftLinear(16, 16, 16, K, 2, 9, 'quantlut_sym', tlut=tl, has_kernel=True)
+    had_l, K_l = mh.get_hadK(k)
+    had_r, K_r = mh.get_hadK(m)
+    out = layer(dev(L["x"]), pk, dev(L["SU"]), dev(L["SV"]), had_l, had_r, K_l, K_r, 0, 8)
+    assert out.dtype == torch.float16 and out.shape == (1, m)
+    ref_l = O.bitshift_linear_forward(L["x"], L["packed"], L["SU"], L["SV"], L["tlut"], K,
+                                      matvec_fn=lambda row: c_oracle.matvec(L["packed"], row, L["tlut"], m, k, K))
+    assert_close(out.cpu().numpy(), ref_l)
+
+
+@pytest.mark.parametrize("m,k", [(28672, 8192), (8192, 28672)])
+def test_batched_product_4bit_at_full_size(m, k):
+    """4-bit weights, batch 8 / 16 / 32: every output against X (float64) times the oracle's
+    decoded matrix; the fp16-rounded form is the rounding of the fp32 one."""
+    from qtip_amd import ops
+    K = 4
+    L = make_layer(m, k, K, seed=m + k)
+    pk, tl = dev(L["packed"]), dev(L["tlut"])
+    w = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float32)  # fp16 values, exact in fp32
+    for batch in (8, 16, 32):
+        X = np.random.default_rng(batch).standard_normal((batch, k)).astype(np.float16)
+        got = ops.decompress_gemm(pk, dev(X), tl, m, k, K, round_f16=False).cpu().numpy()
+        # products of fp16 values are exact in fp32, the sums are taken in float64 blocks
+        ref = np.zeros((batch, m), dtype=np.float64)
+        Xf = X.astype(np.float32)
+        for c0 in range(0, k, 256):
+            ref += (Xf[:, c0:c0 + 256] @ w[:, c0:c0 + 256].T).astype(np.float64)
+        # a block of 256 products summed in fp32 carries <= 256 * 2^-24 relative error: far below the bar
+        assert_close(got, ref)
+        got16 = ops.decompress_gemm(pk, dev(X), tl, m, k, K, round_f16=True).cpu().numpy()
+        assert np.array_equal(got16, got.astype(np.float16).astype(np.float32))
+
+
+def test_full_decoder_7b_architecture():
+    """32 layers, d = 4096, 32 heads, FFN 11008, vocabulary 32000, every projection 2-bit: the
+    fused decode step against the module-by-module forward of the same model (logits and key /
+    value caches), and the captured loop against the eager one, 16 tokens."""
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig()
+    assert (cfg.hidden, cfg.heads, cfg.layers, cfg.ffn, cfg.vocab, cfg.K) == (4096, 32, 32, 11008, 32000, 2)
+    model = LlamaDecoder(cfg, max_cache_len=256)
+    ids = torch.randint(0, cfg.vocab, (1, 24), generator=torch.Generator().manual_seed(0)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(24, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([24], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        vc = [c.clone() for c in model.v_cache]
+        b = model.decode_fused(tok, pos)
+    assert torch.isfinite(a).all() and torch.isfinite(b).all()
+    # 32 layers of fp16 roundings taken at different points: the bar is wider than one layer's
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 5e-2, 1e-2)
+    for c0, c1 in zip(kc + vc, model.k_cache + model.v_cache):
+        assert torch.allclose(c0.float(), c1.float(), atol=5e-2)
+    g, _, _ = generate(model, ids, 16, use_graph=True)
+    e, _, _ = generate(model, ids, 16, use_graph=False)
+    assert g.shape == (1, 16) and torch.equal(g, e)
