@@ -38,6 +38,7 @@ extern "C" {
 #define QTIP_E_ALIGN (-3)     /* a pointer is not 16-byte aligned */
 #define QTIP_E_WORKSPACE (-4) /* workspace smaller than qtip_matvec_workspace_bytes */
 #define QTIP_E_DTYPE (-5)     /* unknown dtype code */
+#define QTIP_E_SCRATCH (-6)   /* partial sums larger than the library's static scratch */
 #define QTIP_E_NOT_INIT (-7)  /* first call on this device came inside a stream capture */
 
 #define QTIP_F16 0
@@ -47,7 +48,8 @@ extern "C" {
 int qtip_abi_version(void);
 
 /* One-time set-up for the CURRENT device: reads the CU count, opts every kernel into its LDS
- * size.  Allocates nothing and does not synchronise.  Idempotent and thread-safe; returns 0 or a hipError_t.  Every launcher
+ * size and looks up the device's copy of the library's static scratch.  Allocates nothing and
+ * does not synchronise.  Idempotent and thread-safe; returns 0 or a hipError_t.  Every launcher
  * runs it on first use of a device, so calling it is only required before a stream capture
  * whose first recorded call would otherwise be the library's first call on that device.
  * No counterpart in the reference (its templates need no run-time set-up). */
@@ -90,6 +92,22 @@ size_t qtip_matvec_workspace_bytes(int m, int k, int bits);
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16,
                            const void* tlut, int m, int k, int bits,
                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* qtip_decompress_matvec for callers that cannot allocate device memory and have no workspace
+ * to pass (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  The split-k partial sums live in a 256 KiB array in the
+ * library's own device image (one copy per GPU, held until the process ends), so the call
+ * allocates nothing: no hipMalloc / hipFree, no workspace argument.
+ *   nparts = 0: the library's choice of k split (the one qtip_decompress_matvec makes with a
+ *               workspace); 1..16: that many k ranges.
+ * Results are bit-identical to qtip_decompress_matvec with the same split.
+ * Limit: nparts * m <= 65536 floats, else QTIP_E_SCRATCH (nothing launched; nparts = 1 never
+ * needs the scratch).  The partial sums are all written before they are read, so nothing has to
+ * be cleared between calls; but every call on a GPU uses that GPU's one array: calls that
+ * overlap in time on one GPU (different streams, or graphs replayed concurrently) race. */
+int qtip_decompress_matvec_noalloc(float* out, const void* packed, const void* x_f16,
+                                   const void* tlut, int m, int k, int bits, int nparts,
+                                   void* stream);
 
 /* Same kernel, but leaves the nparts partial vectors parts[nparts][m] for the
  * consumer to add (qtip_rht does so on load through its in_parts argument),

@@ -44,6 +44,7 @@ _SIGNATURES = {
                                      [ctypes.c_int] * 3 + [ctypes.c_void_p]),
     "qtip_decompress_matvec": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 +
                                [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "qtip_decompress_matvec_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "qtip_gemm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
     "qtip_decompress_gemm": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 +
                              [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),

@@ -997,6 +997,12 @@ __global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict_
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
+// Device memory the allocation-free entry point keeps its split-k partial sums in: one copy per
+// GPU the library runs on, held until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress (never a device address): launches take DeviceState::scratch_ptr.
+constexpr size_t kScratchFloats = 64 * 1024;  // 256 KiB
+static __device__ __align__(256) float scratch[kScratchFloats];
+
 template <typename F>
 hipError_t allow_lds(F* fn, size_t bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
@@ -1041,12 +1047,14 @@ hipError_t allow_lds_all() {
   return hipSuccess;
 }
 
-// Per-device set-up: CU count and LDS opt-in of every kernel.  qtip_init() runs it for the current device; a launcher that meets a device for the
+// Per-device set-up: CU count, LDS opt-in of every kernel, address of this device's copy of
+// `scratch`.  qtip_init() runs it for the current device; a launcher that meets a device for the
 // first time runs it too (none of it allocates or synchronises, but hipFuncSetAttribute is not
 // a call to make while a stream is being captured: callers that record graphs call qtip_init()
 // first).
 struct DeviceState {
   int cus = 0;
+  float* scratch_ptr = nullptr;
   hipError_t status = hipErrorNotInitialized;
   bool done = false;
   bool refused = false;  // first use of the device inside a stream capture: set-up not run
@@ -1086,9 +1094,13 @@ DeviceState& device_state(bool launching = false, hipStream_t st = nullptr) {
   int cus = 0;
   hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (e == hipSuccess) e = allow_lds_all();
+  float* sp = nullptr;
+  if (e == hipSuccess) e = hipGetSymbolAddress(reinterpret_cast<void**>(&sp), HIP_SYMBOL(scratch));
+  if (e == hipSuccess && !sp) e = hipErrorInvalidSymbol;
   d.status = e;
   if (e == hipSuccess) {
     d.cus = cus > 0 ? cus : 256;
+    d.scratch_ptr = sp;
     d.done = true;  // a failed set-up is tried again by the next call
   }
   return d;
@@ -1170,6 +1182,9 @@ const char* qtip_error_string(int code) {
     case QTIP_E_NOT_INIT:
       return "qtip: first call on this device came inside a stream capture; call qtip_init() (or any "
              "launcher) on the device before capturing";
+    case QTIP_E_SCRATCH:
+      return "qtip: the partial sums of this call exceed the library's static scratch (256 KiB); use "
+             "qtip_decompress_matvec with a caller workspace";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "qtip: unknown error";
   }
 }
@@ -1504,6 +1519,25 @@ int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, co
   rc = launch_matvec((float*)workspace, packed, x_f16, tlut, m, k, bits, S, st);
   if (rc) return rc;
   sum_parts_kernel<<<(m + 255) / 256, 256, 0, st>>>(out, (const float*)workspace, m, S);
+  return (int)hipGetLastError();
+}
+
+int qtip_decompress_matvec_noalloc(float* out, const void* packed, const void* x_f16, const void* tlut,
+                                   int m, int k, int bits, int nparts, void* stream) {
+  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits, stream);
+  if (rc) return rc;
+  const DeviceState& ds = device_state();  // set up by check_matvec (or qtip_init) already
+  const int nwl = ((k >> 5) + 3) >> 2;
+  if (nparts < 0 || nparts > kMaxSplit || nparts > nwl) return QTIP_E_SHAPE;
+  const int S = nparts ? nparts : choose_split(m, k, bits, ds.cus, true);
+  hipStream_t st = (hipStream_t)stream;
+  if (S == 1) return launch_matvec(out, packed, x_f16, tlut, m, k, bits, 1, st);
+  if ((size_t)S * m > kScratchFloats) return QTIP_E_SCRATCH;
+  // every one of the S * m partial sums is written before it is read: nothing to clear
+  float* parts = ds.scratch_ptr;
+  rc = launch_matvec(parts, packed, x_f16, tlut, m, k, bits, S, st);
+  if (rc) return rc;
+  sum_parts_kernel<<<(m + 255) / 256, 256, 0, st>>>(out, parts, m, S);
   return (int)hipGetLastError();
 }
 
