@@ -120,6 +120,8 @@ def load_llama(path, max_cache_len=2048, device='cuda'):
     the reference's model (model/llama.py:300-372, 437-531).  Projections in
     quip_params['skip_list'] ('{layer}_{q|k|v|o|up|gate|down}') are dense fp16."""
     cfg, qp = read_config(path)
+    with open(os.path.join(path, 'config.json')) as f:
+        tied = bool(json.load(f).get('tie_word_embeddings', False))
     skip = tuple(qp.get('skip_list') or ())
     model = LlamaDecoder(cfg, max_cache_len, device=device, fused=False, skip=skip, K_v=qp.get('K_v_proj'),
                          random_init=False)
@@ -138,6 +140,12 @@ def load_llama(path, max_cache_len=2048, device='cuda'):
                         raise ValueError(f"{key}: checkpoint shape {tuple(src.shape)}, model {tuple(dst.shape)}")
                     dst.copy_(src.to(dst.dtype))
                     seen.add(key)
+    if tied and 'lm_head.weight' not in seen and 'model.embed_tokens.weight' in seen:
+        # tied output embedding (LlamaForCausalLM._tied_weights_keys, model/llama.py:1350): the file
+        # holds the matrix once, under the embedding's name
+        with torch.no_grad():
+            model.lm_head.copy_(model.embed)
+        seen.add('lm_head.weight')
     missing = sorted(set(targets) - seen)
     if missing:
         raise KeyError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:3]}")

@@ -461,6 +461,10 @@ class _FusedLinear:
         return self.transform_out(self.matvec(self.transform_in(x, pre_mode, norm_weight, eps)), residual)
 
 
+# the decode attention kernel keeps one score per cache slot in LDS
+FUSED_MAX_CACHE_LEN = 4096
+
+
 def _rotate_half(x):
     x1, x2 = x[..., :x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
     return torch.cat((-x2, x1), dim=-1)
@@ -513,8 +517,10 @@ class LlamaDecoder(nn.Module):
 
     def supports_fused_decode(self):
         """False when a layer needs what the fused decode step does not cover (per-shard
-        transforms, rcp != 0, or a layer that is not kernel-packed): generate() then decodes
-        module by module."""
+        transforms, rcp != 0, a layer that is not kernel-packed, or a key / value cache longer than
+        the attention kernel's FUSED_MAX_CACHE_LEN slots): generate() then decodes module by module."""
+        if self.max_cache_len > FUSED_MAX_CACHE_LEN:
+            return False
         try:
             for layer in self.layers:
                 layer._fused_linears()
@@ -526,6 +532,9 @@ class LlamaDecoder(nn.Module):
         """tok (1,1) int64, pos (1,) int64 device tensors -> logits (1, 1, vocab), fused kernels;
         fp32 as the reference returns them, or the fp16 values the lm_head product yields
         (float_logits=False, what the greedy pick reads)."""
+        if self.max_cache_len > FUSED_MAX_CACHE_LEN:
+            raise ValueError(f"the fused decode step covers caches of up to {FUSED_MAX_CACHE_LEN} slots "
+                             f"(this model has {self.max_cache_len}); decode module by module")
         x = self.embed[tok.reshape(-1)]
         qp = None
         for i, layer in enumerate(self.layers):
@@ -565,6 +574,12 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
     the streaming hook of the interactive script; reading the value synchronises."""
     dev = prompt_ids.device
     n = prompt_ids.shape[1]
+    # the last token that is fed back sits at position n + max_new_tokens - 2; past the cache the
+    # fused kernels would silently drop its key / value (the position is device memory, nothing
+    # on the host sees it), so the whole request is checked here
+    if n < 1 or n + max(max_new_tokens, 1) - 1 > model.max_cache_len:
+        raise ValueError(f"prompt of {n} tokens + {max_new_tokens} new tokens does not fit the key / value cache "
+                         f"of {model.max_cache_len} slots")
     sampling = temperature is not None
     fused = fused and model.supports_fused_decode()
 

@@ -22,13 +22,15 @@ _SPLIT = {}
 
 
 def _workspace(device, need):
+    """Scratch of at least `need` bytes for the current stream.  A request beyond the current
+    buffer gets a larger one, and the smaller ones stay alive for the life of the process: a
+    HIP graph recorded earlier still holds their addresses."""
     dev = device.index if device.index is not None else torch.cuda.current_device()
     key = (dev, torch.cuda.current_stream(device).cuda_stream)
-    ws = _WORKSPACE.get(key)
-    if ws is None or ws.numel() < need:
-        ws = torch.empty(max(need, _WORKSPACE_BYTES), dtype=torch.uint8, device=device)
-        _WORKSPACE[key] = ws
-    return ws
+    held = _WORKSPACE.setdefault(key, [])
+    if not held or held[-1].numel() < need:
+        held.append(torch.empty(max(need, _WORKSPACE_BYTES), dtype=torch.uint8, device=device))
+    return held[-1]
 
 
 def matvec_split(m, k, bits, device):

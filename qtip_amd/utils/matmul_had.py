@@ -73,14 +73,23 @@ def had_bits(hadK, K, transpose, device):
             neg = _table_signs(K).astype(bool)
             _bit_cache[key] = torch.from_numpy(_pack_bits(neg.T if transpose else neg)).to(dev)
         return _bit_cache[key]
-    key = (hadK.data_ptr(), hadK._version, tuple(hadK.shape), tuple(hadK.stride()), bool(transpose), dev)
-    if key not in _bit_cache:
+    # a caller's own table: the cache entry keeps the tensor alive, so its address cannot be handed to
+    # another tensor while the entry exists, and remembers the version it was packed from
+    key = (hadK.data_ptr(), tuple(hadK.shape), tuple(hadK.stride()), bool(transpose), dev)
+    hit = _bit_cache.get(key)
+    if hit is None or hit[0] is not hadK or hit[1] != hadK._version:
         h = hadK.detach().to("cpu", torch.float32).numpy()
         if h.shape != (K, K) or not np.all(np.abs(h) == 1.0):
             raise ValueError("hadK must be a K x K matrix of +-1")
         neg = h < 0
-        _bit_cache[key] = torch.from_numpy(_pack_bits(neg.T if transpose else neg)).to(dev)
-    return _bit_cache[key]
+        # a K x K table equal to the built-in one shares the built-in entry
+        if K in _ORDERS and np.array_equal(neg, _table_signs(K).astype(bool)):
+            bits = had_bits(None, K, transpose, dev)
+        else:
+            bits = torch.from_numpy(_pack_bits(neg.T if transpose else neg)).to(dev)
+        hit = (hadK, hadK._version, bits)
+        _bit_cache[key] = hit
+    return hit[2]
 
 
 _dense_cache = {}

@@ -9,8 +9,10 @@ imported or executed), extracts the +1/-1 literals of every `get_hadN`
 function and stores them as packed bits (bit set = -1), 15 KB in total.
 
 Run once in a container that has the reference checkout:
-    python qtip_amd/utils/make_hadamard_tables.py [/root/reference]
-The .npz it writes is committed; nothing reads the reference at run time.
+    python tests/golden/make_hadamard_tables.py [/root/reference]
+The .npz it writes (qtip_amd/utils/hadamard_tables.npz) is committed; nothing reads the reference
+at run time.  tests/golden/had_digests.json (make_had_digests.py, an independent parse of the same
+literals) pins its contents.
 """
 import os
 import re
@@ -48,7 +50,8 @@ def main():
     if missing:
         raise SystemExit(f"missing orders {missing}")
     out = {f"had{o}": np.packbits((tables[o] < 0).astype(np.uint8).reshape(-1)) for o in ORDERS}
-    dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "hadamard_tables.npz")
+    root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    dst = os.path.join(root, "qtip_amd", "utils", "hadamard_tables.npz")
     np.savez(dst, **out)
     print("wrote", dst, {k: v.size for k, v in out.items()})
 

@@ -114,6 +114,94 @@ def test_unpack_quip_folds_wscale(rcp):
         assert int(lin.rcp) == rcp and int(lin.tp_rank) == shards
 
 
+def _reference_schema_checkpoint(tmp_path, tie=False):
+    """A checkpoint written WITHOUT this package's key map: the keys come from
+    tests/golden/checkpoint_keys.json (derived from the text of the reference's model/llama.py and
+    lib/linear/quantized_linear.py by tests/golden/make_checkpoint_keys.py), the shapes and dtypes
+    from QuantizedLinear's constructor in the reference (lib/linear/quantized_linear.py:41-67)."""
+    from safetensors.torch import save_file
+    schema = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'checkpoint_keys.json')))
+    ex = schema['example']
+    hidden, heads, kv_heads, ffn, vocab, K = 256, 4, 2, 512, 96, 2
+    kvd = hidden // heads * kv_heads
+    dims = {'q_proj': (hidden, hidden), 'k_proj': (hidden, kvd), 'v_proj': (hidden, kvd), 'o_proj': (hidden, hidden),
+            'gate_proj': (hidden, ffn), 'up_proj': (hidden, ffn), 'down_proj': (ffn, hidden)}
+    g = torch.Generator().manual_seed(5)
+    tensors = {}
+    for key in ex['keys']:
+        parts = key.split('.')
+        leaf, owner = parts[-1], parts[-2]
+        if owner in dims:
+            fin, fout = dims[owner]
+            if leaf == 'trellis':
+                t = torch.randint(-32768, 32768, (fout // 16 * (fin // 16), 16 * K), dtype=torch.int16, generator=g)
+            elif leaf == 'tlut':
+                t = torch.randn(512, 2, generator=g).half()
+            elif leaf == 'SU':
+                t = torch.sign(torch.randn(fin, generator=g) + 1e-5).half()
+            elif leaf == 'SV':
+                t = torch.sign(torch.randn(fout, generator=g) + 1e-5) * 0.05
+            elif leaf == 'rcp':
+                t = torch.tensor(0)
+            elif leaf == 'tp_rank':
+                t = torch.tensor(8)
+            elif leaf == 'weight':  # a projection named in skip_list: dense nn.Linear (out, in)
+                t = (torch.randn(fout, fin, generator=g) * 0.05).half()
+            else:
+                raise AssertionError(key)
+        elif owner in ('embed_tokens', 'lm_head'):
+            t = (torch.randn(vocab, hidden, generator=g) * 0.02).half()
+        else:  # RMSNorm weights
+            t = (torch.rand(hidden, generator=g) + 0.5).half()
+        tensors[key] = t
+    if tie:
+        del tensors['lm_head.weight']
+    # a buffer older transformers versions wrote and newer ones do not (non-persistent in the reference)
+    tensors['model.layers.0.self_attn.rotary_emb.inv_freq'] = torch.ones(hidden // heads // 2)
+    save_file(tensors, str(tmp_path / 'model.safetensors'), metadata={'format': 'pt'})
+    config = dict(model_type='llama', hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                  num_hidden_layers=ex['num_hidden_layers'], intermediate_size=ffn, vocab_size=vocab,
+                  rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=tie,
+                  quip_params=dict(td_x=16, td_y=16, L=16, K=K, V=2, tlut_bits=9, decode_mode='quantlut_sym',
+                                   skip_list=ex['skip_list']))
+    json.dump(config, open(tmp_path / 'config.json', 'w'))
+    return ex, tensors
+
+
+@pytest.mark.parametrize("tie", [False, True])
+def test_loader_reads_the_reference_key_schema(tmp_path, tie):
+    ex, tensors = _reference_schema_checkpoint(tmp_path, tie)
+    model = C.load_llama(str(tmp_path), max_cache_len=64, device='cpu')
+    # the loader's own key map names exactly the reference's state-dict keys
+    assert set(C._targets(model)) == set(ex['keys'])
+    # and every tensor sits where the reference's module tree puts it
+    l0, l1 = model.layers
+    t = lambda k: tensors[k]
+    assert torch.equal(l0.q_proj.trellis, t('model.layers.0.self_attn.q_proj.trellis'))
+    assert torch.equal(l0.v_proj.SU, t('model.layers.0.self_attn.v_proj.SU'))
+    assert torch.equal(l0.o.SV, t('model.layers.0.self_attn.o_proj.SV'))
+    assert torch.equal(l0.gate_proj.tlut.data, t('model.layers.0.mlp.gate_proj.tlut'))
+    assert torch.equal(l1.up_proj.trellis, t('model.layers.1.mlp.up_proj.trellis'))
+    assert torch.equal(l1.down.SV, t('model.layers.1.mlp.down_proj.SV'))
+    assert isinstance(l1.k_proj, torch.nn.Linear) and torch.equal(l1.k_proj.weight, t('model.layers.1.self_attn.k_proj.weight'))
+    assert isinstance(l0.down, torch.nn.Linear) and torch.equal(l0.down.weight, t('model.layers.0.mlp.down_proj.weight'))
+    assert torch.equal(l0.input_norm.weight, t('model.layers.0.input_layernorm.weight'))
+    assert torch.equal(l1.post_norm.weight, t('model.layers.1.post_attention_layernorm.weight'))
+    assert torch.equal(model.norm.weight, t('model.norm.weight'))
+    assert torch.equal(model.embed, t('model.embed_tokens.weight'))
+    assert torch.equal(model.lm_head, t('model.embed_tokens.weight' if tie else 'lm_head.weight'))
+    assert int(l0.q_proj.rcp) == 0 and int(l0.q_proj.tp_rank) == 8
+
+
+def test_untied_checkpoint_without_lm_head_is_incomplete(tmp_path):
+    _reference_schema_checkpoint(tmp_path, tie=True)
+    cfg = json.load(open(tmp_path / 'config.json'))
+    cfg['tie_word_embeddings'] = False
+    json.dump(cfg, open(tmp_path / 'config.json', 'w'))
+    with pytest.raises(KeyError):
+        C.load_llama(str(tmp_path), 64, 'cpu')
+
+
 @pytest.mark.gpu
 def test_loaded_model_runs_like_the_original(tmp_path):
     from qtip_amd.llama_decode import generate

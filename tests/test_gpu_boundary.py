@@ -54,3 +54,39 @@ def test_first_call_inside_a_capture_is_a_defined_error_then_init_and_capture_wo
     """) % ROOT
     res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0 and "ok" in res.stdout, res.stdout + res.stderr
+
+
+def test_workspace_growth_keeps_the_buffer_a_recorded_graph_writes_to():
+    """A graph recorded with the split-k workspace of the moment keeps working after a later,
+    larger request replaced that workspace: the old buffer stays allocated."""
+    import numpy as np
+    import torch
+    from oracle import c_oracle
+    from qtip_amd import ops
+    from synth import make_layer
+    m, k, K = 128, 28672, 2
+    L = make_layer(m, k, K, seed=3)
+    pk, x, tl = (torch.from_numpy(np.ascontiguousarray(L[n])).cuda() for n in ("packed", "x", "tlut"))
+    x = x.reshape(-1)
+    out = torch.zeros(m, device="cuda")
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        ops.decompress_matvec(pk, x, tl, m, k, K, out=out)  # eager first: allocations happen here
+        torch.cuda.synchronize()
+        eager = out.clone()
+        held = ops._WORKSPACE[(pk.device.index, s.cuda_stream)]
+        n_before, old = len(held), held[-1]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            ops.decompress_matvec(pk, x, tl, m, k, K, out=out)
+        bigger = ops._workspace(pk.device, old.numel() + 1)
+        assert bigger.numel() > old.numel() and len(held) == n_before + 1 and held[-2] is old
+        filler = [torch.full((old.numel(),), 0x7F, dtype=torch.uint8, device="cuda") for _ in range(4)]
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+        del filler
+    ref = c_oracle.matvec(L["packed"], L["x"].reshape(-1), L["tlut"], m, k, K)
+    assert np.abs(eager.double().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()

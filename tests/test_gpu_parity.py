@@ -227,6 +227,24 @@ def test_bitshift_linear_forward(m, n, K, bs):
     assert_close(out.cpu().numpy(), ref)
 
 
+def test_layer_rounds_the_matmul_result_to_fp16_only_for_more_than_one_row():
+    """The hand-built case of synth.rounding_case on the device: 6.0 for one row (fp32 matvec), 8.0
+    for two (the batched product's result passes through fp16, lib/codebook/bitshift.py:476-489)."""
+    from qtip_amd.codebook.bitshift import BitshiftLinear
+    from synth import rounding_case
+    L = rounding_case()
+    layer = BitshiftLinear(16, 16, 16, 2, 2, 9, 'quantlut_sym', tlut=dev(L["tlut"]), has_kernel=True)
+    args = (dev(L["packed"]), dev(L["SU"]), dev(L["SV"]), None, None, 1, 1, 0, 8)
+    one = layer(dev(L["x"]), *args).cpu().numpy()
+    assert float(one[0, 0]) == 6.0 and float(one[0, 16]) == 16384.0 and np.count_nonzero(one) == 2
+    two = layer(dev(np.repeat(L["x"], 2, axis=0)), *args).cpu().numpy()
+    assert float(two[0, 0]) == 8.0 and float(two[1, 0]) == 8.0 and np.count_nonzero(two) == 4
+    for bs, want in ((1, 6.0), (2, 8.0), (40, 8.0)):
+        ref = O.bitshift_linear_forward(np.repeat(L["x"], bs, axis=0), L["packed"], L["SU"], L["SV"], L["tlut"], 2)
+        got = layer(dev(np.repeat(L["x"], bs, axis=0)), *args).cpu().numpy()
+        assert float(got[0, 0]) == want and np.array_equal(got, ref)
+
+
 def test_bitshift_linear_matches_dense_equivalent():
     # the reference's own dense form of the layer (bitshift.py:389-413)
     from qtip_amd.codebook.bitshift import BitshiftLinear

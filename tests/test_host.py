@@ -222,3 +222,21 @@ def test_bench_refuses_more_than_one_gpu():
                        text=True, timeout=120)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_generate_refuses_requests_beyond_the_cache():
+    """The fused decode step keeps its position in device memory and would silently drop keys past
+    the cache; the request is checked on the host before anything runs."""
+    from qtip_amd.llama_decode import FUSED_MAX_CACHE_LEN, LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=256, heads=4, kv_heads=2, layers=1, ffn=512, vocab=64)
+    model = LlamaDecoder(cfg, max_cache_len=16, device="cpu")
+    ids = torch.zeros((1, 10), dtype=torch.int64)
+    with pytest.raises(ValueError, match="does not fit"):
+        generate(model, ids, 8)  # positions up to 16 needed, slots 0..15 exist
+    with pytest.raises(ValueError, match="does not fit"):
+        generate(model, torch.zeros((1, 17), dtype=torch.int64), 1)
+    assert model.supports_fused_decode()
+    long = LlamaDecoder(cfg, max_cache_len=FUSED_MAX_CACHE_LEN + 1, device="cpu")
+    assert not long.supports_fused_decode()  # generate() then decodes module by module
+    with pytest.raises(ValueError, match="fused decode step covers"):
+        long.decode_fused(torch.zeros((1, 1), dtype=torch.int64), torch.tensor([0]))

@@ -179,6 +179,57 @@ def test_known_table_rows():
     assert sym == {12: False, 20: False, 28: True, 172: False}
 
 
+def test_tables_match_the_reference_literals():
+    """Every order-K table against tests/golden/had_digests.json: sha256 of the table as the
+    reference writes it (lib/utils/matmul_had.py:129-95715), taken by an `ast` parse of that file
+    (tests/golden/make_had_digests.py) independent of the reader that produced the .npz.  A row
+    permutation, a transposition or a flipped sign changes the digest."""
+    import hashlib
+    import json
+    import os
+    import torch
+    from qtip_amd.utils import matmul_had as mh
+    gold = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "had_digests.json")))
+    assert sorted(v["order"] for v in gold.values()) == [12, 20, 28, 36, 52, 60, 108, 116, 124, 140, 156, 172]
+    for name, g in gold.items():
+        o = g["order"]
+        h = O._load_tables()[o]
+        assert hashlib.sha256(h.astype(np.int8).tobytes()).hexdigest() == g["sha256"], name
+        assert h[0].astype(int).tolist() == g["row0"] and int(h[:, 0].sum()) == g["col0_sum"]
+        assert bool(np.array_equal(h, h.T)) == g["symmetric"]
+        # the product's own reader of the same file
+        hp = 1.0 - 2.0 * mh._table_signs(o).astype(np.float64)
+        assert hashlib.sha256(hp.astype(np.int8).tobytes()).hexdigest() == g["sha256"], name
+        had, K = mh.get_hadK(o * 8)
+        if K == o:  # orders that a larger order does not shadow at this size
+            assert hashlib.sha256(had.numpy().astype(np.int8).tobytes()).hexdigest() == g["sha256"]
+        hadT, _ = mh.get_hadK(o * 8, transpose=True)
+        if K == o:
+            assert torch.equal(hadT, had.T)
+
+
+def test_layer_rounds_the_matmul_result_to_fp16_only_for_more_than_one_row():
+    """Hand-built case (synth.rounding_case): output element 0 is 6.0 from the fp32 matvec of a
+    single row and 8.0 once the matmul result passes through fp16, as the reference's batched path
+    does (lib/codebook/bitshift.py:443-448 against :476-489)."""
+    from synth import rounding_case
+    L = rounding_case()
+    idx, sign = O.hyb_hash(np.array([0x0000, 0x1111]))
+    assert idx.tolist() == [0, 336] and sign.tolist() == [0, 0]
+    w = O.decode_kernel(L["packed"], L["tlut"], 64, 64, 2).astype(np.float64)
+    for r in range(64):
+        want = (64.0, 3.0 / 64.0) if r % 32 < 16 else (-64.0, 0.0)
+        assert np.all(w[r, 0::2] == want[0]) and np.all(w[r, 1::2] == want[1])
+    one, parts = O.bitshift_linear_forward(L["x"], L["packed"], L["SU"], L["SV"], L["tlut"], 2, return_parts=True)
+    assert np.all(parts["x4"] == 1.0)
+    assert set(np.unique(parts["y0"]).tolist()) == {2049.5, -2048.0}
+    assert float(one[0, 0]) == 6.0 and float(one[0, 16]) == 16384.0
+    assert np.count_nonzero(one) == 2
+    two = O.bitshift_linear_forward(np.repeat(L["x"], 2, axis=0), L["packed"], L["SU"], L["SV"], L["tlut"], 2)
+    assert two.shape == (2, 64) and float(two[0, 0]) == 8.0 and float(two[1, 0]) == 8.0
+    assert float(two[0, 16]) == 16384.0 and np.count_nonzero(two) == 4
+
+
 @pytest.mark.parametrize("n,order", [(11008, 172), (12288, 12), (10240, 20), (28672, 28), (22016, 172),
                                      (57344, 28), (4096, 1), (8192, 1)])
 def test_get_hadK_factorisation(n, order):
