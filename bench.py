@@ -19,6 +19,9 @@ Prints ONE JSON line:  value = packed bytes streamed per second (GB/s), plus
   decode_dense  packed -> dense fp16 weights: time, GB/s written, (read + written) / 8 TB/s
   measured_ceilings  copy / fill / sum bandwidth of this box (library kernels) beside the nominal peak
   e2e_decode    greedy decode tok/s of a random-init 7B-architecture 2-bit model
+  sets          the other matvec sets: Llama-2-7B shapes at 2 / 3 / 4 bits, 70B shapes at 3 / 4 bits
+                (set GB/s and per-matrix times, cold weights)
+  single_layer  one 4096x4096 2-bit BitshiftLinear: kernel and whole forward, cold and cache-resident
 """
 import argparse
 import json
@@ -30,9 +33,37 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch over algorithmic bytes per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this script, each calibrated against a 256 MiB copy (summary under profiles/)
-MEASURED_TRAFFIC_RATIO = {("70b", 2): (52583.0 + 82.0) / 52224.0}
+# HBM bytes per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each calibrated
+# against a 256 MiB copy) are read from this summary, which names the kernel sources it was taken on
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "matvec_k2_llama70b_set_traffic.txt")
+KERNEL_SOURCES = ("qtip_amd/csrc/qtip_hip.hip", "qtip_amd/csrc/qtip_device.h", "qtip_amd/csrc/qtip_wht.h")
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, bits):
+    """(bytes per launch or None, note): the counter-measured HBM traffic of the headline kernel, only
+    if the committed summary was taken on exactly the kernel sources of this tree."""
+    if (workload, bits) != ("70b", 2):
+        return None, "no counter profile for this workload"
+    try:
+        kv = dict(line.split(":", 1) for line in open(TRAFFIC_FILE) if ":" in line and not line.startswith("#"))
+        kv = {k.strip(): v.strip() for k, v in kv.items()}
+    except OSError:
+        return None, "profiles/matvec_k2_llama70b_set_traffic.txt not present where this ran"
+    if kv.get("kernel_source_digest") != kernel_source_digest():
+        return None, "the committed counter profile was taken on older kernel sources; not carried over"
+    return int(kv["traffic_bytes_per_launch"]), "FETCH_SIZE + WRITE_SIZE per launch, rocprofv3 --pmc, see " + \
+        os.path.relpath(TRAFFIC_FILE, ROOT)
+
+
 SHAPES_70B = [("qkv", 10240, 8192), ("o", 8192, 8192), ("up_gate", 57344, 8192), ("down", 8192, 28672)]
 SHAPES_7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("up_gate", 22016, 4096), ("down", 4096, 11008)]
 
@@ -58,13 +89,18 @@ def main():
                          "counter runs under rocprofv3")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip per-shape / layer / GEMM / end-to-end timings")
-    ap.add_argument("--extras", default="shapes,layer,gemm,decode,ceilings,e2e",
-                    help="comma-separated subset of the extra sections to run: shapes, layer, gemm, decode, ceilings, e2e, e2e13b, e2e70b "
-                         "(counter runs under rocprofv3 pick one)")
+    ap.add_argument("--extras", default="shapes,layer,sets,single,gemm,decode,ceilings,e2e",
+                    help="comma-separated subset of the extra sections to run: shapes, layer, sets, single, gemm, decode, "
+                         "ceilings, e2e, e2e13b, e2e70b (counter runs under rocprofv3 pick one)")
+    ap.add_argument("--print-kernel-source-digest", action="store_true",
+                    help="print the digest that profiles/matvec_k2_llama70b_set_traffic.txt must name, and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs)")
     args = ap.parse_args()
+    if args.print_kernel_source_digest:
+        print(kernel_source_digest())
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (--gpus 1); no multi-GPU figure is produced",
               file=sys.stderr)
@@ -165,6 +201,7 @@ def main():
     avg_launch_us = dev_s * 1e6 / launches
     achieved = (set_bytes / len(shapes)) / (avg_launch_us * 1e-6) / 1e9
 
+    traffic, traffic_note = measured_traffic(args.workload, K)
     result = {
         "metric": "bs=1 2-bit decompress-matvec compressed-stream throughput, Llama-2-70B layer shapes",
         "value": round(value, 1),
@@ -197,9 +234,8 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "avg_launch_us": round(avg_launch_us, 3),
             "bytes_per_launch": set_bytes // len(shapes),
-            "traffic": (round(MEASURED_TRAFFIC_RATIO[(args.workload, K)] * set_bytes / len(shapes))
-                        if (args.workload, K) in MEASURED_TRAFFIC_RATIO and args.shape is None else None),
-            "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, see profiles/)",
+            "traffic": traffic if args.shape is None else None,
+            "traffic_note": traffic_note,
         },
         "host_wall_s_timed_region": round(wall_s, 4),
     }
@@ -236,6 +272,83 @@ def main():
             del gr, pks
         result["shapes"] = per
         result["layer"] = layer
+
+    def cold_copies(base, nbytes):
+        """Enough distinct copies of one matrix to cycle through more than twice the 256 MB last-level
+        cache, so that every launch streams from HBM."""
+        ncp = max(2, -(-(600 << 20) // nbytes))
+        return [base] + [torch.roll(base, 4099 * c) for c in range(1, ncp)]
+
+    if "sets" in extras:
+        # the matvec sets the headline does not cover: 7B shapes at every bit width, 70B at 3 and 4 bits
+        sets = {}
+        for wl, shp, bits_list in (("7b", SHAPES_7B, (2, 3, 4)), ("70b", SHAPES_70B, (3, 4))):
+            for kb in bits_list:
+                if (wl, kb) == (args.workload, K):
+                    continue
+                sb = sum(m * k * kb // 8 for _, m, k in shp)
+                ncp = max(2, -(-(600 << 20) // sb))
+                pk, xv, ov = {}, {}, {}
+                for name, m, k in shp:
+                    base = torch.randint(-32768, 32768, (m * k * kb // 16,), dtype=torch.int16, generator=g).to(dev)
+                    pk[name] = [base] + [torch.roll(base, 4099 * c) for c in range(1, ncp)]
+                    xv[name] = torch.randn(k, generator=g).half().to(dev)
+                    ov[name] = torch.empty(m, dtype=torch.float32, device=dev)
+                nst = max(args.steps, 2 * ncp)
+                gr = capture(lambda: [ops.decompress_matvec(pk[name][i % ncp], xv[name], tlut, m, k, kb, out=ov[name])
+                                      for i in range(nst) for name, m, k in shp])
+                st_s = timed(gr, 1, args.settle_ms) / nst
+                del gr
+                entry = {"GBps": round(sb / st_s / 1e9, 1), "frac_hbm_peak": round(sb / st_s / 1e9 / HBM_PEAK_GBS, 4),
+                         "ms_per_step": round(st_s * 1e3, 5), "bytes_per_step": sb, "shapes": {}}
+                for name, m, k in shp:
+                    nbytes = m * k * kb // 8
+                    pks = pk[name] + [torch.roll(pk[name][0], 4099 * c)
+                                      for c in range(ncp, max(ncp, -(-(600 << 20) // nbytes)))]
+                    reps = len(pks) * max(1, 24 // len(pks))
+                    gr = capture(lambda: [ops.decompress_matvec(pks[i % len(pks)], xv[name], tlut, m, k, kb,
+                                                               out=ov[name]) for i in range(reps)])
+                    us = timed(gr, 3, args.settle_ms / 3) * 1e6 / reps
+                    entry["shapes"][name] = {"m": m, "k": k, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                                             "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                    del gr, pks
+                sets[f"{wl}_k{kb}"] = entry
+                del pk, xv, ov
+                torch.cuda.empty_cache()
+        result["sets"] = sets
+
+    if "single" in extras:
+        # one BitshiftLinear, 4096 x 4096, 2 bits: the kernel alone and the whole forward (input transform
+        # inside the matvec launch + output transform), with cold weights (copies rotated through more than
+        # twice the last-level cache) and with one cache-resident copy
+        from qtip_amd.codebook.bitshift import BitshiftLinear
+        from qtip_amd.utils import matmul_had as mh
+        m = k = 4096
+        nbytes = m * k * 2 // 8
+        base = torch.randint(-32768, 32768, (m * k * 2 // 16,), dtype=torch.int16, generator=g).to(dev)
+        pks = cold_copies(base, nbytes)
+        xv = torch.randn(k, generator=g).half().to(dev)
+        ov = torch.empty(m, dtype=torch.float32, device=dev)
+        mod = BitshiftLinear(16, 16, 16, 2, 2, 9, "quantlut_sym", tlut=tlut, has_kernel=True)
+        SU = torch.sign(torch.randn(k, generator=g) + 1e-5).half().to(dev)
+        SV = (torch.sign(torch.randn(m, generator=g) + 1e-5) / k**0.5).float().to(dev)
+        inp = torch.randn(1, k, generator=g).half().to(dev)
+        single = {"m": m, "k": k, "bits": 2, "packed_bytes": nbytes, "weight_copies_rotated": len(pks)}
+        for label, pool in (("cold", pks), ("warm", pks[:1])):
+            reps = max(len(pool), 150)
+            gr = capture(lambda: [ops.decompress_matvec(pool[i % len(pool)], xv, tlut, m, k, 2, out=ov)
+                                  for i in range(reps)])
+            us = timed(gr, 3, args.settle_ms / 3) * 1e6 / reps
+            del gr
+            gr = capture(lambda: [mod(inp, pool[i % len(pool)].view(-1, 32), SU, SV, None, None, 1, 1, 0, 8)
+                                  for i in range(reps)])
+            lus = timed(gr, 3, args.settle_ms / 3) * 1e6 / reps
+            del gr
+            single[label] = {"kernel_us": round(us, 2), "kernel_GBps": round(nbytes / us / 1e3, 1),
+                             "kernel_frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "forward_us": round(lus, 2), "forward_GBps": round(nbytes / lus / 1e3, 1)}
+        result["single_layer_4096x4096_k2"] = single
+        del pks, base
 
     if "gemm" in extras:
         # batched decompress-GEMM on the matrix cores: 4-bit weights, batch 8 / 16 / 32
@@ -295,9 +408,14 @@ def main():
         model = LlamaDecoder(LlamaConfig(K=2), max_cache_len=512, device=dev)
         prompt = torch.randint(0, 32000, (1, 128), generator=g).to(dev)
         toks, dt, tps = generate(model, prompt, 256, use_graph=True, fused=True)
+        # bytes a decoded token must read: every packed matrix, the fp16 lm_head and the keys / values so far
+        tok_bytes = sum(l.trellis.numel() * 2 for l in model.modules() if hasattr(l, "trellis")) + \
+            model.lm_head.numel() * 2 + 2 * 32 * (128 + 128) * 4096 * 2
         result["e2e_decode"] = {"model": "Llama-2-7B architecture, random init, 2-bit HYB, fused qkv and up/gate",
                                 "prompt": 128, "new_tokens": 256, "tok_per_s": round(tps, 1),
-                                "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 256)}
+                                "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 256),
+                                "bytes_per_token": tok_bytes,
+                                "frac_hbm": round(tok_bytes * tps / 1e9 / HBM_PEAK_GBS, 4)}
         del model
         torch.cuda.empty_cache()
         # the layout of the published checkpoints: seven separate projections per layer (grouped launches)
