@@ -186,7 +186,11 @@ template <int K>
 __device__ __forceinline__ LaneData<K> load_lane_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff,
                                                      uint32_t soff) {
   LaneData<K> r;
-  constexpr int NT = 2;  // non-temporal: the stream is read once
+  // Non-temporal where a load instruction covers whole cache lines (one 16-byte load per lane at 2
+  // bits) or nearly so (3 bits): the stream is read once.  At 4 bits a lane's two 16-byte loads
+  // split every line between two instructions, and with the hint the second one fetches the line
+  // from L2 again: plain loads are 10 % faster there (57344x8192: 47.7 -> 41.5 us).
+  constexpr int NT = K == 4 ? 0 : 2;
   if constexpr (K == 2) {
     const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, NT);
 #pragma unroll
@@ -983,6 +987,284 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// 4-bit batched decompress + GEMM on a row-split lane map: no product is computed twice
+// ---------------------------------------------------------------------------
+// In gemm_kernel the two lanes that share a matrix row hold different column halves of it, which
+// costs every product twice (and 64 accumulator registers for 32 batch rows, hence 8 waves).
+// Here the two lanes of a pair load the SAME 64 bytes - the four reference lanes of one row of a
+// 2x2 tile block, i.e. all 16 columns of that row in each of the four tiles - and split the
+// STATES: a 32-bit chunk holds four states, the even lane decodes states 0 and 2 (rows r), the
+// odd lane states 1 and 3 (rows r + 8).  A byte permutation with a per-lane selector puts the
+// lane's two states of a chunk into one register, so the decode costs what it costs in
+// gemm_kernel (32 lookups per lane and wave-load).  The 16 lanes of a DPP row now hold the same
+// 8 columns of 16 different rows: a v_mfma_f32_16x16x32_f16 B operand whose every output is
+// wanted.  Per wave-load and 16 batch rows: 8 products instead of 16, 8 accumulator registers
+// instead of 32, so 32 batch rows run on the 16-wave workgroup (4 waves per SIMD).
+// Lane (g, a): tile block g of the wave-load, row r = a / 2 (+ 8 for odd a) of either tile row
+// half; registers D[cp][t]: reference lane 4 r + cp (columns 2 cp, 2 cp + 1 of an 8-column
+// group), tile t = 2 kh + mh.  The successor chunk of cp = 3 sits two lanes on (row r + 1, the
+// ring of 32 reference lanes closing inside the 16-lane row).
+// The two lanes of a pair read the same bytes and the four 16-byte loads of a lane walk the same
+// cache lines, so the loads are plain (cached) ones: with the non-temporal hint of the other
+// kernels every load instruction fetched its lines from L2 again (43 us instead of 29 us at batch
+// 8).  HBM traffic is unchanged.
+// One activation tile (16 NB batch rows x 1024 columns) in LDS, single-buffered: the next tile
+// waits in registers while the current one is used, two barriers per stage.
+constexpr int kGemm4Waves = 16, kGemm4KS = 4;
+constexpr size_t kGemm4TileBytes = 32 * 1024;
+constexpr size_t kGemm4Lds = kLut128Bytes + kGemm4TileBytes;
+
+template <int NB>
+__global__ __launch_bounds__(kThreads, 1) void gemm4_kernel(
+    float* __restrict__ dst, const uint8_t* __restrict__ packed, const uint16_t* __restrict__ x,
+    const uint32_t* __restrict__ tlut, int m, int k, int batch, int round_f16, int wl_per, int upw_q,
+    int upw_r) {
+  constexpr int K = 4, DEPTH = 2, KS = kGemm4KS;
+  constexpr int ROWB = KS * 256;  // bytes per tile row
+  constexpr int CPR = ROWB / 16;  // 16-byte chunks per tile row
+  constexpr uint32_t TILE = 16 * NB * ROWB;
+  constexpr bool DB = 2 * TILE <= kGemm4TileBytes;  // room for two tiles: one barrier per stage instead of two
+  static_assert(TILE <= kGemm4TileBytes, "tile does not fit");
+  static_assert(16 * NB * CPR == NB * kThreads, "NB chunks per thread and tile");
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+  uint8_t* tile = smem + kLut128Bytes;  // [1 or 2][16*NB rows][ROWB bytes]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rbi = wave & (kGemmRB - 1), ks = wave >> 2;
+  const int a = lane & 15, g = lane >> 4;
+  const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
+  const int nkb = k >> 5;
+  const int nwl = (nkb + 3) >> 2;
+  const int nrb = m >> 5;
+  const int ngroups = (nrb + kGemmRB - 1) / kGemmRB;
+  const uint32_t rb_bytes = (uint32_t)nkb * 128 * K;
+  constexpr uint32_t WL_BYTES = 512 * K;
+  const uint32_t loff = (uint32_t)g * (128 * K) + (uint32_t)(a >> 1) * (16 * K);  // the row's four reference lanes
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(packed), 0, (int)((size_t)nrb * rb_bytes), 0x00020000);
+  // states 0 | 2 of a chunk for even lanes (the chunk as it is), 1 | 3 for odd lanes (chunk bytes
+  // 2 1 | chunk byte 0, successor byte 3)
+  const uint32_t sel = (a & 1) ? 0x06050403u : 0x07060504u;
+
+  const int s = blockIdx.x;
+  const int g0 = blockIdx.y, gstep = gridDim.y;
+  const int wl0 = s * wl_per;  // wl_per is a multiple of KS
+  const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
+  const int nst = wl1 > wl0 ? (wl1 - wl0 + KS - 1) / KS : 0;  // stages per unit
+  const int upw = upw_q + (g0 < upw_r ? 1 : 0);
+  const int T = upw * nst;
+  float* out_s = dst + (size_t)s * batch * m;
+
+  struct Raw {
+    uint32_t d[4][4];  // [cp][t]
+  };
+  int l_t = 0, l_q = 0, l_grp = g0;
+  Raw buf[DEPTH];
+  auto issue = [&](int d) {
+    const int rb = l_grp * kGemmRB + rbi;
+    const int wl = wl0 + KS * l_t + ks;
+    const bool valid = l_q < T && rb < nrb && wl < wl1;
+    const uint32_t vo = valid ? loff : 0x7FFFFF00u;  // padding: out of range, no memory access
+    const uint32_t so = valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u;
+#pragma unroll
+    for (int cp = 0; cp < 4; ++cp) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, vo + 16 * cp, so, 0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) buf[d].d[cp][t] = v[t];
+    }
+    ++l_q;
+    if (++l_t == nst) {
+      l_t = 0;
+      l_grp += gstep;
+    }
+  };
+  // table words through the scalar cache first, one stage of the stream before the table is built
+  uint32_t tw[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t* tp = tlut + j * 128 + wave * 8;
+    uint32_t v = tp[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) v = ((lane >> 3) == e) ? tp[e] : v;
+    tw[j] = v;
+  }
+  issue(0);
+
+  static_assert(DEPTH % 2 == 0, "stage parity must be static inside the unrolled loop");
+  u32x4 xg[2][NB];  // tiles on their way: [parity of the stage][chunk], requested two stages ahead
+  auto load_tile = [&](int slot, int t) {  // stage t of a unit -> registers
+    const int col0 = 128 * (wl0 + KS * t);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int idx = i * kThreads + tid;
+      const int b = idx / CPR, c = idx % CPR;
+      const int col = col0 + 8 * c;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (b < batch && col < k) v = *reinterpret_cast<const u32x4*>(x + (size_t)b * k + col);
+      xg[slot][i] = v;
+    }
+  };
+  // registers -> LDS buffer (the buffer of the stage's parity when there are two), chunk index
+  // xor-ed with the row: conflict-free both ways
+  auto store_tile = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int idx = i * kThreads + tid;
+      const int b = idx / CPR, c = idx % CPR;
+      *reinterpret_cast<u32x4*>(tile + (DB ? slot * TILE : 0u) + b * ROWB + ((c ^ (b & 7)) << 4)) = xg[slot][i];
+    }
+  };
+  load_tile(0, 0);
+  load_tile(1, nst > 1 ? 1 : 0);
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const uint32_t w = tw[it & 3] ^ ((uint32_t)(it >> 2) << 15);
+    const u32x4 v = {w, w, w, w};
+    reinterpret_cast<u32x4*>(lut)[it * kThreads + tid] = v;
+  }
+  store_tile(0);
+  __syncthreads();
+  issue(1);
+
+  float4_t acc[2][NB];  // [mh][batch tile]
+#pragma unroll
+  for (int i = 0; i < 2 * NB; ++i) (&acc[0][0])[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+  uint32_t arow[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) arow[nb] = (uint32_t)(16 * nb + a) * ROWB;
+  const uint32_t a7 = (uint32_t)(a & 7);
+  const uint32_t tile_addr = lds_address(tile);
+  typedef __attribute__((address_space(3))) const u32x4 lds_u32x4_t;
+
+  int c_t = 0, c_grp = g0;
+  for (int q = 0; q < T; q += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const bool live = q + d < T;  // uniform over the workgroup
+      if (live) {
+        const int rb = c_grp * kGemmRB + rbi;
+        const int wl = wl0 + KS * c_t + ks;
+        if (rb < nrb && wl < wl1) {
+          const Raw& R = buf[d];
+          const uint32_t tb = tile_addr + (DB ? (uint32_t)((q + d) & 1) * TILE : 0u);
+          uint32_t W[4][4][2];  // [cp][t][jh]
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            // successor of reference lane 4 r + 3: reference lane 4 (r + 1), two lanes on in the row
+            const uint32_t nx = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)R.d[0][t], 0x12E /* row_ror:14 */,
+                                                                      0xF, 0xF, false);
+#pragma unroll
+            for (int cp = 0; cp < 4; ++cp) {
+              const uint32_t c = R.d[cp][t];
+              const uint32_t cn = cp < 3 ? R.d[cp + 1][t] : nx;
+              const uint32_t P = perm(c, cn, sel);  // high half: state 0 or 1, low half: state 2 or 3
+              const uint32_t hq = pk_hash(P) & 0xFFC0FFC0u;
+              W[cp][t][0] = lds_word_abs(lut128_addr_hi(hq, slot4));
+              W[cp][t][1] = lds_word_abs(lut128_addr_lo(hq, slot4));
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+            for (int jh = 0; jh < 2; ++jh) {
+              u32x4 xa[NB];
+              const uint32_t c = (uint32_t)(16 * ks + 4 * g + 2 * kh + jh) ^ a7;
+#pragma unroll
+              for (int nb = 0; nb < NB; ++nb)
+                xa[nb] = *(lds_u32x4_t*)(uintptr_t)(tb + arow[nb] + (c << 4));
+#pragma unroll
+              for (int mh = 0; mh < 2; ++mh) {
+                const int t = 2 * kh + mh;
+                const u32x4 wv = {W[0][t][jh], W[1][t][jh], W[2][t][jh], W[3][t][jh]};
+                const half8_t bop = __builtin_bit_cast(half8_t, wv);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                  acc[mh][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa[nb]), bop,
+                                                                       acc[mh][nb], 0, 0, 0);
+              }
+            }
+        }
+      }
+      issue(d);
+      if (live) {
+        if constexpr (DB) {
+          // the next tile (in registers since the previous stage) into the other buffer, the one
+          // after it on its way (slot = parity of that stage = parity of this one)
+          store_tile((q + d + 1) & 1);
+          int t2 = c_t + 2;
+          if (t2 >= nst) t2 -= nst;
+          if (t2 >= nst) t2 -= nst;  // nst == 1
+          load_tile((q + d) & 1, t2);
+        }
+        __syncthreads();  // every wave has read this stage's tile (and, with two buffers, written the next)
+        const int rb = c_grp * kGemmRB + rbi;
+        if (++c_t == nst) {
+          // ---- end of a unit: the k slices of a row block meet in the tile buffer (free between the
+          // two barriers of a stage): slices 1 .. KS-1 hand their sums over in turn, the wave of
+          // slice 0 adds them in that order, rounds and stores
+          float* xch = reinterpret_cast<float*>(tile + (DB ? (uint32_t)((q + d) & 1) * TILE : 0u)) + rbi * (64 * 8 * NB);
+          float4_t vals[2][NB];
+#pragma unroll
+          for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              vals[mh][nb] = acc[mh][nb];
+              acc[mh][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+          for (int turn = 1; turn < KS; ++turn) {
+            if (ks == turn) {
+#pragma unroll
+              for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                  *reinterpret_cast<float4_t*>(xch + ((mh * NB + nb) * 64 + lane) * 4) = vals[mh][nb];
+            }
+            __syncthreads();
+            if (ks == 0) {
+#pragma unroll
+              for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                  const float4_t o = *reinterpret_cast<const float4_t*>(xch + ((mh * NB + nb) * 64 + lane) * 4);
+                  vals[mh][nb] += o;
+                }
+            }
+            __syncthreads();
+          }
+          if (ks == 0 && rb < nrb) {
+#pragma unroll
+            for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+              for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                  float sum = vals[mh][nb][i];
+                  if (round_f16) sum = (float)(_Float16)sum;
+                  // lane (g, a): batch row 16*nb + 4*g + i, matrix row 16*mh + 8*(a%2) + a/2
+                  const int bb = 16 * nb + 4 * g + i;
+                  if (bb < batch) out_s[(size_t)bb * m + rb * 32 + 16 * mh + 8 * (a & 1) + (a >> 1)] = sum;
+                }
+          }
+          c_t = 0;
+          c_grp += gstep;
+        }
+        if constexpr (!DB) {
+          // one buffer: the next tile (in registers since the previous stage) goes in now, the one
+          // after it on its way (slot = parity of that stage = parity of this one)
+          store_tile((q + d + 1) & 1);
+          int t2 = c_t + 1;
+          if (t2 >= nst) t2 -= nst;
+          load_tile((q + d) & 1, t2);
+          __syncthreads();  // the next tile is complete
+        }
+      }
+    }
+  }
+}
+
 // out[i] = parts[0][i] + ... (+ rounding through fp16) for the split-k GEMM
 __global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict__ out,
                                                               const float* __restrict__ parts, long n,
@@ -1043,6 +1325,8 @@ hipError_t allow_lds_all() {
   QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
   QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
   QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
+  QTIP_ALLOW((gemm4_kernel<1>), kGemm4Lds)
+  QTIP_ALLOW((gemm4_kernel<2>), kGemm4Lds)
 #undef QTIP_ALLOW
   return hipSuccess;
 }
@@ -1586,7 +1870,12 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   // up to 16 rows run on the 16-wave workgroup (4 wave-loads per stage)
   for (int b0 = 0; b0 < batch; b0 += 32) {
     const int nb = batch - b0 < 32 ? batch - b0 : 32;
-    const int KS = nb <= 16 ? 4 : 2;
+#ifndef QTIP_NO_GEMM4
+    const bool rowsplit = bits == 4;  // the 4-bit kernel without duplicated products, 16 waves for every batch
+#else
+    const bool rowsplit = false;
+#endif
+    const int KS = (rowsplit || nb <= 16) ? 4 : 2;
     int Sp = S;
     int wl_per = (nwl + Sp - 1) / Sp;
     wl_per = (wl_per + KS - 1) / KS * KS;  // stages are groups of KS wave-loads
@@ -1606,10 +1895,19 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
 #define QTIP_GEMM_K(KB)               \
   if (nb <= 16) QTIP_GEMM(KB, 1, 16); \
   else QTIP_GEMM(KB, 2, 8);
-    switch (bits) {
-      case 2: QTIP_GEMM_K(2) break;
-      case 3: QTIP_GEMM_K(3) break;
-      default: QTIP_GEMM_K(4) break;
+    if (rowsplit) {
+      if (nb <= 16)
+        gemm4_kernel<1><<<g2, kThreads, kGemm4Lds, st>>>(d, p, xx, t, m, k, nb, rnd, wl_per, ngroups / per_range,
+                                                         ngroups % per_range);
+      else
+        gemm4_kernel<2><<<g2, kThreads, kGemm4Lds, st>>>(d, p, xx, t, m, k, nb, rnd, wl_per, ngroups / per_range,
+                                                         ngroups % per_range);
+    } else {
+      switch (bits) {
+        case 2: QTIP_GEMM_K(2) break;
+        case 3: QTIP_GEMM_K(3) break;
+        default: QTIP_GEMM_K(4) break;
+      }
     }
 #undef QTIP_GEMM_K
 #undef QTIP_GEMM
