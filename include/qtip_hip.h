@@ -270,10 +270,17 @@ int qtip_rht_chain(void* xt_out_f16, void* x_out_f16, const float* parts, int in
  * token's position (model/cache_utils.py:1173-1193), softmax(q K^T / sqrt(d)) V over cache slots
  * 0..pos (model/llama.py:866-880).  qkv_f16 = [heads*d | kv_heads*d | kv_heads*d] of the new token,
  * caches are [kv_heads][max_len][d] fp16, pos_i64 points to the position in DEVICE memory (a
- * recorded graph then follows the position), inv_freq[d/2] fp32.  out_f16 = [heads*d]. */
+ * recorded graph then follows the position), inv_freq[d/2] fp32.  out_f16 = [heads*d].
+ * key_splits (1..16): 1 = one workgroup per head walks the whole context (right up to a few
+ * hundred keys: 6 us at 128, 10 us at 1024, 28 us at 4095); > 1 = the cache slots are cut into
+ * key_splits equal ranges of max_len / key_splits slots, one workgroup per head and range, and a
+ * second small launch combines the ranges' softmax shares, which pass through split_workspace:
+ * heads * key_splits * (head_dim + 2) floats, 16-byte aligned, no initialisation needed (may be
+ * NULL when key_splits == 1).  The caller picks key_splits from the longest context the call (or
+ * the graph it records) will see. */
 int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16, void* v_cache_f16,
                           const void* pos_i64, const float* inv_freq, int heads, int kv_heads,
-                          int head_dim, int max_len, void* stream);
+                          int head_dim, int max_len, int key_splits, float* split_workspace, void* stream);
 
 /* qtip_decode_attention on the qkv projection's raw matvec result: the output transform of
  * BitshiftLinear.forward (lib/codebook/bitshift.py:465-472: H_R, then * SV * 32) runs in the
@@ -289,7 +296,7 @@ int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, s
                               const float* post_f32, float scale, const uint32_t* had_bits, int order,
                               void* k_cache_f16, void* v_cache_f16, const void* pos_i64,
                               const float* inv_freq, int heads, int kv_heads, int head_dim, int max_len,
-                              void* stream);
+                              int key_splits, float* split_workspace, void* stream);
 
 /* qtip_decode_attention_rht for separate q / k / v projections: three raw matvec results, each
  * with the output transform of its own QuantizedLinear (q: heads * head_dim elements, k and v:
@@ -301,7 +308,8 @@ int qtip_decode_attention_rht3(void* out_f16, const float* const* parts, int in_
                                const float* const* post_f32, const float* scale,
                                const uint32_t* const* had_bits, const int* order, void* k_cache_f16,
                                void* v_cache_f16, const void* pos_i64, const float* inv_freq, int heads,
-                               int kv_heads, int head_dim, int max_len, void* stream);
+                               int kv_heads, int head_dim, int max_len, int key_splits,
+                               float* split_workspace, void* stream);
 
 /* Final RMSNorm of the decoder for one vector: out = weight * fp16(x * rsqrt(mean(x^2) + eps))
  * (model/llama.py:129-135), n <= 16384, one launch instead of the module's six. */

@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 _lib = None
 
@@ -67,12 +67,12 @@ _SIGNATURES = {
     "qtip_rht_chain": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_float,
                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
                                       ctypes.c_float, ctypes.c_void_p]),
-    "qtip_decode_attention": (ctypes.c_int, [ctypes.c_void_p] * 6 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
+    "qtip_decode_attention": (ctypes.c_int, [ctypes.c_void_p] * 6 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "qtip_decode_attention_rht": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_int, ctypes.c_size_t,
                                                  ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_int] +
-                                  [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
+                                  [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "qtip_decode_attention_rht3": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_int, ctypes.c_size_t] +
-                                   [ctypes.c_void_p] * 8 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
+                                   [ctypes.c_void_p] * 8 + [ctypes.c_int] * 5 + [ctypes.c_void_p] * 2),
     "qtip_rmsnorm": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_float, ctypes.c_int, ctypes.c_void_p]),
     "qtip_greedy_pick": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3 +
                          [ctypes.c_long, ctypes.c_long, ctypes.c_void_p]),

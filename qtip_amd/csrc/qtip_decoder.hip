@@ -53,14 +53,20 @@ struct AttnXf {
 
 typedef float float4a __attribute__((ext_vector_type(4)));
 
-// One workgroup per query head.  qkv: [H*D | Hkv*D | Hkv*D] fp16 of the new
+// One workgroup per query head and key range.  qkv: [H*D | Hkv*D | Hkv*D] fp16 of the new
 // token; k_cache / v_cache: [Hkv][max_len][D] fp16; pos_ptr: position of the
 // new token (device memory, so that a recorded graph follows the position).
+// nsplit > 1 (long contexts): workgroup blockIdx.z takes the keys
+// [z * keys_per_split, (z + 1) * keys_per_split) and leaves its share - the D unnormalised output
+// sums, its score maximum and its sum of exponentials - in split_ws[head][z][D + 2] for
+// attn_combine_kernel; every workgroup repeats the prologue (transform, rotary embedding), the
+// one of range 0 writes the cache.
 template <int D, int XF>
 __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     _Float16* __restrict__ out, const _Float16* __restrict__ qkv, _Float16* __restrict__ k_cache,
     _Float16* __restrict__ v_cache, const long* __restrict__ pos_ptr,
-    const float* __restrict__ inv_freq, int H, int Hkv, int max_len, const AttnXf X) {
+    const float* __restrict__ inv_freq, int H, int Hkv, int max_len, const AttnXf X, int nsplit,
+    int keys_per_split, float* __restrict__ split_ws) {
   extern __shared__ __align__(16) uint8_t smem[];
   float* q_s = reinterpret_cast<float*>(smem);   // [D] rotated query (as fp16 values)
   float* k_s = q_s + kMaxHeadDim;                // [D] rotated new key
@@ -308,7 +314,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
     q_s[tid] = (float)qe;
     k_s[tid] = (float)ke;
     v_s[tid] = (float)v0;
-    if (blockIdx.x == 0 && pos < max_len) {
+    if (blockIdx.x == 0 && blockIdx.z == 0 && pos < max_len) {
       kc[(size_t)pos * D + tid] = ke;
       vc[(size_t)pos * D + tid] = v0;
     }
@@ -318,17 +324,19 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   // ---- scores: 8 lanes per key (16 dims each), 128 keys per pass
   const float sm_scale = rsqrtf((float)D);
   const int nkeys = pos + 1 < max_len ? pos + 1 : max_len;
+  const int k0 = (int)blockIdx.z * keys_per_split;                       // this workgroup's keys: [k0, k1)
+  const int k1 = k0 + keys_per_split < nkeys ? k0 + keys_per_split : nkeys;
   const int sub = tid & 7, kq = tid >> 3;
   constexpr int dper = D >> 3;  // dims per lane (multiple of 8: D % 64 == 0)
   float mx = -INFINITY;
   // four keys per thread group and round, all of their loads issued before the first use
   constexpr int KU = 4;
-  for (int t0 = 0; t0 < nkeys; t0 += KU * (kAttnThreads / 8)) {
+  for (int t0 = k0; t0 < k1; t0 += KU * (kAttnThreads / 8)) {
     uint4 raw[KU][dper / 8];
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
       const int t = t0 + kq + u * (kAttnThreads / 8);
-      const int tc = (t < nkeys && t != pos) ? t : 0;  // clamped: the new key comes from LDS
+      const int tc = (t < k1 && t != pos) ? t : 0;  // clamped: the new key comes from LDS
       const uint4* kr = reinterpret_cast<const uint4*>(kc + (size_t)tc * D + sub * dper);
 #pragma unroll
       for (int d8 = 0; d8 < dper / 8; ++d8) raw[u][d8] = kr[d8];
@@ -351,8 +359,8 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
       s += qtip_wht::lane_xor(s, 1);
       s += qtip_wht::lane_xor(s, 2);
       s *= sm_scale;
-      if (t < nkeys) {
-        if (sub == 0) p_s[t] = s;
+      if (t < k1) {
+        if (sub == 0) p_s[t - k0] = s;
         mx = fmaxf(mx, s);
       }
     }
@@ -366,8 +374,8 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
   uint4 vfirst[VU];
 #pragma unroll
   for (int u = 0; u < VU; ++u) {
-    const int t = tg + u * TG;
-    const int tc = (t < nkeys && t != pos) ? t : 0;
+    const int t = k0 + tg + u * TG;
+    const int tc = (t < k1 && t != pos) ? t : 0;
     vfirst[u] = *reinterpret_cast<const uint4*>(vc + (size_t)tc * D + dg * 8);
   }
   mx = wave_reduce_max(mx);
@@ -377,7 +385,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
 #pragma unroll
   for (int w = 1; w < 16; ++w) mx = fmaxf(mx, red[w]);
   float sum = 0.f;
-  for (int t = tid; t < nkeys; t += kAttnThreads) {
+  for (int t = tid; t < k1 - k0; t += kAttnThreads) {
     const float e = __expf(p_s[t] - mx);
     p_s[t] = e;
     sum += e;
@@ -393,24 +401,24 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
 
   // ---- output: thread (tg, dg) sums keys tg, tg+TG, ... for dims 8*dg .. 8*dg+7
   float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int t0 = tg; t0 < nkeys; t0 += VU * TG) {
+  for (int t0 = k0 + tg; t0 < k1; t0 += VU * TG) {
     uint4 raw[VU];
-    if (t0 == tg) {
+    if (t0 == k0 + tg) {
 #pragma unroll
       for (int u = 0; u < VU; ++u) raw[u] = vfirst[u];
     } else {
 #pragma unroll
       for (int u = 0; u < VU; ++u) {
         const int t = t0 + u * TG;
-        const int tc = (t < nkeys && t != pos) ? t : 0;
+        const int tc = (t < k1 && t != pos) ? t : 0;
         raw[u] = *reinterpret_cast<const uint4*>(vc + (size_t)tc * D + dg * 8);
       }
     }
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
       const int t = t0 + u * TG;
-      if (t < nkeys) {
-        const float pt = p_s[t];
+      if (t < k1) {
+        const float pt = p_s[t - k0];
         if (t == pos) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) o[e] += pt * v_s[dg * 8 + e];
@@ -441,24 +449,57 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attn_kernel(
       acc[tid] = tot2;  // only read by this thread below
     }
   }
-  if (tid < D) out[(size_t)h * D + tid] = (_Float16)(acc[tid] * inv);
+  if (nsplit == 1) {
+    if (tid < D) out[(size_t)h * D + tid] = (_Float16)(acc[tid] * inv);
+  } else if (tid < D) {
+    float* w = split_ws + ((size_t)h * nsplit + blockIdx.z) * (D + 2);
+    w[tid] = acc[tid];  // 0 for a range past the last key
+    if (tid == 0) {
+      w[D] = mx;        // -inf for an empty range
+      w[D + 1] = tot;
+    }
+  }
+}
+
+// out[head] = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z over the key ranges of a head
+// (M = max_z m_z): the softmax of the whole context from the shares of its ranges.
+__global__ __launch_bounds__(kMaxHeadDim) void attn_combine_kernel(_Float16* __restrict__ out,
+                                                                  const float* __restrict__ split_ws,
+                                                                  int nsplit, int D) {
+  const int h = blockIdx.x, d = threadIdx.x;
+  const float* w = split_ws + (size_t)h * nsplit * (D + 2);
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, w[z * (D + 2) + D]);
+  float num = 0.f, den = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float mz = w[z * (D + 2) + D];
+    const float e = mz == -INFINITY ? 0.f : __expf(mz - M);
+    num += e * w[z * (D + 2) + d];
+    den += e * w[z * (D + 2) + D + 1];
+  }
+  out[(size_t)h * D + d] = (_Float16)(num / den);
 }
 
 }  // namespace
 
 static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf, int xf_mode, void* k_cache_f16,
                             void* v_cache_f16, const void* pos_i64, const float* inv_freq, int heads,
-                            int kv_heads, int head_dim, int max_len, void* stream) {
+                            int kv_heads, int head_dim, int max_len, int key_splits, float* split_ws,
+                            void* stream) {
   if (!out_f16 || !k_cache_f16 || !v_cache_f16 || !pos_i64 || !inv_freq) return QTIP_E_NULL;
+  if (key_splits < 1 || key_splits > 16) return QTIP_E_SHAPE;
+  if (key_splits > 1 && !split_ws) return QTIP_E_NULL;
+  if (key_splits > 1 && (reinterpret_cast<uintptr_t>(split_ws) & 15)) return QTIP_E_ALIGN;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads || head_dim < 64 || head_dim > kMaxHeadDim ||
       (head_dim & (head_dim - 1)) || max_len < 1 || max_len > 4096)
     return QTIP_E_SHAPE;
   const size_t lds = (size_t)(3 * kMaxHeadDim + 32 + 8192 + max_len) * sizeof(float);
-  const dim3 grid((unsigned)(heads / kv_heads), (unsigned)kv_heads);
+  const dim3 grid((unsigned)(heads / kv_heads), (unsigned)kv_heads, (unsigned)key_splits);
+  const int kps = (max_len + key_splits - 1) / key_splits;  // keys per range
 #define QTIP_ATTN(DD, XX, ARG)                                                                      \
   decode_attn_kernel<DD, XX><<<grid, kAttnThreads, lds, (hipStream_t)stream>>>(                      \
       (_Float16*)out_f16, (const _Float16*)qkv_f16, (_Float16*)k_cache_f16, (_Float16*)v_cache_f16,  \
-      (const long*)pos_i64, inv_freq, heads, kv_heads, max_len, ARG)
+      (const long*)pos_i64, inv_freq, heads, kv_heads, max_len, ARG, key_splits, kps, split_ws)
   if (xf) {
     if (head_dim != 64 && head_dim != 128) return QTIP_E_SHAPE;
     if (xf_mode == 1) {
@@ -474,6 +515,10 @@ static int launch_attention(void* out_f16, const void* qkv_f16, const AttnXf* xf
     }
   }
 #undef QTIP_ATTN
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || key_splits == 1) return (int)e;
+  attn_combine_kernel<<<heads, head_dim, 0, (hipStream_t)stream>>>((_Float16*)out_f16, split_ws, key_splits,
+                                                                   head_dim);
   return (int)hipGetLastError();
 }
 
@@ -498,17 +543,19 @@ static int fill_xf_slot(AttnXf& x, int slot, const float* parts, const float* po
 
 extern "C" int qtip_decode_attention(void* out_f16, const void* qkv_f16, void* k_cache_f16,
                                      void* v_cache_f16, const void* pos_i64, const float* inv_freq,
-                                     int heads, int kv_heads, int head_dim, int max_len, void* stream) {
+                                     int heads, int kv_heads, int head_dim, int max_len, int key_splits,
+                                     float* split_workspace, void* stream) {
   if (!qkv_f16) return QTIP_E_NULL;
   return launch_attention(out_f16, qkv_f16, nullptr, 0, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads,
-                          kv_heads, head_dim, max_len, stream);
+                          kv_heads, head_dim, max_len, key_splits, split_workspace, stream);
 }
 
 extern "C" int qtip_decode_attention_rht(void* out_f16, const float* parts, int in_parts, size_t part_stride,
                                          const float* post_f32, float scale, const uint32_t* had_bits,
                                          int order, void* k_cache_f16, void* v_cache_f16,
                                          const void* pos_i64, const float* inv_freq, int heads,
-                                         int kv_heads, int head_dim, int max_len, void* stream) {
+                                         int kv_heads, int head_dim, int max_len, int key_splits,
+                                         float* split_workspace, void* stream) {
   if (in_parts < 1 || in_parts > 16 || heads < 1 || kv_heads < 1 || head_dim < 64 || head_dim > 128 ||
       (part_stride & 3))
     return QTIP_E_SHAPE;
@@ -519,14 +566,15 @@ extern "C" int qtip_decode_attention_rht(void* out_f16, const float* parts, int 
   x.part_stride = part_stride;
   x.in_parts = in_parts;
   return launch_attention(out_f16, nullptr, &x, 1, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
-                          head_dim, max_len, stream);
+                          head_dim, max_len, key_splits, split_workspace, stream);
 }
 
 extern "C" int qtip_decode_attention_rht3(void* out_f16, const float* const* parts, int in_parts,
                                           size_t part_stride, const float* const* post_f32, const float* scale,
                                           const uint32_t* const* had_bits, const int* order, void* k_cache_f16,
                                           void* v_cache_f16, const void* pos_i64, const float* inv_freq,
-                                          int heads, int kv_heads, int head_dim, int max_len, void* stream) {
+                                          int heads, int kv_heads, int head_dim, int max_len, int key_splits,
+                                          float* split_workspace, void* stream) {
   if (!parts || !post_f32 || !scale || !had_bits || !order) return QTIP_E_NULL;
   if (in_parts < 1 || in_parts > 16 || heads < 1 || kv_heads < 1 || head_dim < 64 || head_dim > 128 ||
       (part_stride & 3))
@@ -540,7 +588,7 @@ extern "C" int qtip_decode_attention_rht3(void* out_f16, const float* const* par
   x.part_stride = part_stride;
   x.in_parts = in_parts;
   return launch_attention(out_f16, nullptr, &x, 2, k_cache_f16, v_cache_f16, pos_i64, inv_freq, heads, kv_heads,
-                          head_dim, max_len, stream);
+                          head_dim, max_len, key_splits, split_workspace, stream);
 }
 
 // ---- token head of the decode loop: final RMSNorm and the greedy pick ------------------------

@@ -1451,7 +1451,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 18; }
+int qtip_abi_version(void) { return 19; }
 
 int qtip_init(void) { return (int)device_state().status; }
 

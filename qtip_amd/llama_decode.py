@@ -34,6 +34,9 @@ class LlamaConfig:
         self.ffn, self.vocab, self.rope_theta, self.eps, self.K = ffn, vocab, rope_theta, eps, K
         self.head_dim = hidden // heads
         self.rope_scaling = dict(rope_scaling) if rope_scaling else None
+        # key ranges per head of the fused decode attention; generate() sets it from the longest
+        # context the run will reach (ops.attention_key_splits)
+        self.attn_key_splits = 1
 
 
 def rope_inv_freq(cfg):
@@ -200,10 +203,10 @@ class DecoderLayer(nn.Module):
             # the attention kernel transforms the head-sized slices it needs itself
             q = f['qkv']
             attn = ops.decode_attention_rht(qkv_parts, q.SV, (q.m**-0.5) * 32.0, q.br, q.Kr, k_cache, v_cache, pos,
-                                            inv_freq, cfg.heads, cfg.kv_heads, cfg.head_dim)
+                                            inv_freq, cfg.heads, cfg.kv_heads, cfg.head_dim, key_splits=cfg.attn_key_splits)
         else:
             attn = ops.decode_attention(qkv.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
-                                        cfg.head_dim)
+                                        cfg.head_dim, key_splits=cfg.attn_key_splits)
         if self.fused and f['o'].can_chain_into(f['up_gate']):
             parts = f['o'].matvec_from(attn.reshape(1, -1))
             x, ug_parts = f['o'].chain_matvec(parts, x, f['up_gate'], self.post_norm.weight, cfg.eps)
@@ -302,7 +305,7 @@ class DecoderLayer(nn.Module):
             off += l.m
         attn = ops.decode_attention_rht3(views, [l.SV for l in qkv], [(l.m**-0.5) * 32.0 for l in qkv],
                                          [l.br for l in qkv], [l.Kr for l in qkv], k_cache, v_cache, pos, inv_freq,
-                                         cfg.heads, cfg.kv_heads, cfg.head_dim)
+                                         cfg.heads, cfg.kv_heads, cfg.head_dim, key_splits=cfg.attn_key_splits)
         x = f['o'](attn.reshape(1, -1), residual=x)
         gu_parts = self._group_plain(('gate_proj', 'up_proj'), x, self._su_gate_up, self.post_norm.weight)
         h, pre = self._gate_up_out(gu_parts)
@@ -342,7 +345,7 @@ class DecoderLayer(nn.Module):
         if qkv_parts is None:  # first layer: no boundary in front of it
             vec = torch.cat([l(x, ops.PRE_RMSNORM, self.input_norm.weight, cfg.eps) for l in qkv], dim=-1)
             attn = ops.decode_attention(vec.reshape(-1), k_cache, v_cache, pos, inv_freq, cfg.heads, cfg.kv_heads,
-                                        cfg.head_dim)
+                                        cfg.head_dim, key_splits=cfg.attn_key_splits)
         else:
             views, off = [], 0
             for l in qkv:
@@ -350,7 +353,7 @@ class DecoderLayer(nn.Module):
                 off += l.m
             attn = ops.decode_attention_rht3(views, [l.SV for l in qkv], [(l.m**-0.5) * 32.0 for l in qkv],
                                              [l.br for l in qkv], [l.Kr for l in qkv], k_cache, v_cache, pos, inv_freq,
-                                             cfg.heads, cfg.kv_heads, cfg.head_dim)
+                                             cfg.heads, cfg.kv_heads, cfg.head_dim, key_splits=cfg.attn_key_splits)
         po = f['o'].matvec_from(attn.reshape(1, -1))
         gu_parts, x = self._group_chain(('gate_proj', 'up_proj'), po, f['o'], x, self.post_norm.weight)
         h, pre = self._gate_up_out(gu_parts)
@@ -618,8 +621,9 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
         lg = model.decode_fused(static_tok, static_pos) if fused else model(static_tok, static_pos)
         return lg if sampling else pick(lg)
 
-    graph = None
-    if use_graph:
+    def capture():
+        """Two eager steps (allocations, set-up), then the step recorded into a graph; the decode
+        state is put back afterwards, so a capture in the middle of a run leaves it untouched."""
         keep = (static_tok.clone(), static_pos.clone(), history.clone(), draw_counter.clone())
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -632,18 +636,39 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
                     history.copy_(keep[2])
                     draw_counter.copy_(keep[3])
         torch.cuda.current_stream().wait_stream(s)
-        # the warm-up wrote cache slot n with this token's k/v, which the timed step rewrites identically
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            static_next = step()
+        # the warm-up wrote the cache slot of the current position with this token's k/v, which the
+        # next step rewrites identically
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            nxt = step()
         if on_device:  # capture only records; restore in case the stream ran anything
             static_tok.copy_(keep[0])
             static_pos.copy_(keep[1])
             history.copy_(keep[2])
             draw_counter.copy_(keep[3])
+        return g, nxt
+
+    # the fused attention has two forms (one workgroup per head; key ranges for long contexts): a run
+    # that crosses ops.ATTN_SPLIT_FROM records its step again there, so short contexts never pay
+    # for the second launch of the long form
+    splits_at = lambda ctx: ops.attention_key_splits(ctx) if fused else 1
+    model.cfg.attn_key_splits = splits_at(n + 1)
+    graph = static_next = None
+    if use_graph:
+        graph, static_next = capture()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    recapture_s = 0.0
     for i in range(max_new_tokens - 1):
+        want = splits_at(n + i + 1)  # this step attends to n + i + 1 cache slots
+        if want != model.cfg.attn_key_splits:
+            model.cfg.attn_key_splits = want
+            if graph is not None:
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                graph, static_next = capture()
+                torch.cuda.synchronize()
+                recapture_s += time.perf_counter() - t1  # recording is set-up, not decoding
         if graph is not None:
             graph.replay()
             nxt = static_next
@@ -661,7 +686,7 @@ def generate(model, prompt_ids, max_new_tokens, use_graph=True, fused=True, temp
         if callback is not None:
             callback(out[-1])
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    dt = time.perf_counter() - t0 - recapture_s
     if on_device:
         return history[:max_new_tokens].view(1, -1).clone(), dt, (max_new_tokens - 1) / dt
     return torch.cat(out, dim=1), dt, (max_new_tokens - 1) / dt

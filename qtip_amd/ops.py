@@ -430,7 +430,29 @@ def rht_silu_pair_ok(n, order, two_vectors):
     return pp >= 8
 
 
-def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head_dim):
+ATTN_MAX_KEY_SPLITS = 16
+
+
+ATTN_SPLIT_FROM = 1024  # context length from which the key-range form is faster
+
+
+def attention_key_splits(context):
+    """Key ranges per head for decode attention over a context of `context` tokens: one workgroup
+    per head below ATTN_SPLIT_FROM keys (the ranges cost a second small launch: 32 heads of 128,
+    127 keys 5.8 vs 11.5 us), 8 ranges from there on (2047 keys 22.8 -> 12.9 us, 4095 keys
+    40 -> 20.6 us, which is the time the 67 MB of keys and values take to arrive)."""
+    return 1 if context < ATTN_SPLIT_FROM else 8
+
+
+def _split_workspace(device, heads, head_dim, key_splits):
+    if not 1 <= key_splits <= ATTN_MAX_KEY_SPLITS:
+        raise ValueError(f"key_splits must be in 1..{ATTN_MAX_KEY_SPLITS} (got {key_splits})")
+    if key_splits == 1:
+        return None
+    return torch.empty(heads * key_splits * (head_dim + 2), dtype=torch.float32, device=device)
+
+
+def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head_dim, key_splits=1):
     """Attention output (heads*head_dim,) fp16 of one new token: RoPE, cache write at `pos`
     (device int64 tensor with one element) and attention over cache slots 0..pos in one launch.
     k_cache / v_cache: (1, kv_heads, max_len, head_dim) fp16, updated in place."""
@@ -444,15 +466,16 @@ def decode_attention(qkv, k_cache, v_cache, pos, inv_freq, heads, kv_heads, head
             or v_cache.shape != k_cache.shape or inv_freq.numel() != head_dim // 2 or pos.numel() != 1:
         raise ValueError("decode_attention: inconsistent shapes")
     out = torch.empty(heads * head_dim, dtype=torch.float16, device=qkv.device)
+    ws = _split_workspace(qkv.device, heads, head_dim, key_splits)
     with torch.cuda.device(qkv.device):
         check(lib().qtip_decode_attention(_ptr(out), _ptr(qkv), _ptr(k_cache), _ptr(v_cache), _ptr(pos),
-                                          _ptr(inv_freq), heads, kv_heads, head_dim, max_len,
+                                          _ptr(inv_freq), heads, kv_heads, head_dim, max_len, key_splits, _ptr(ws),
                                           stream_ptr(qkv.device)), "qtip_decode_attention")
     return out
 
 
 def decode_attention_rht(parts, post, scale, had_bits, order, k_cache, v_cache, pos, inv_freq, heads, kv_heads,
-                         head_dim):
+                         head_dim, key_splits=1):
     """decode_attention on the qkv projection's raw matvec result `parts` (S, n) fp32: the
     projection's output transform (order x power-of-two Hadamard, * post * scale, cast to fp16) runs
     in the attention kernel's prologue.  had_bits: the table's packed sign bits (None for order 1)."""
@@ -473,18 +496,20 @@ def decode_attention_rht(parts, post, scale, had_bits, order, k_cache, v_cache, 
             or (order > 1 and had_bits is None):
         raise ValueError("decode_attention_rht: inconsistent shapes")
     out = torch.empty(heads * head_dim, dtype=torch.float16, device=parts.device)
+    ws = _split_workspace(parts.device, heads, head_dim, key_splits)
     with torch.cuda.device(parts.device):
         check(lib().qtip_decode_attention_rht(_ptr(out), _ptr(parts), parts.shape[0], parts.stride(0),
                                               _ptr(post) if post is not None else None, float(scale),
                                               _ptr(had_bits) if had_bits is not None else None, int(order),
                                               _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(inv_freq), heads,
-                                              kv_heads, head_dim, max_len, stream_ptr(parts.device)),
+                                              kv_heads, head_dim, max_len, key_splits, _ptr(ws),
+                                              stream_ptr(parts.device)),
               "qtip_decode_attention_rht")
     return out
 
 
 def decode_attention_rht3(parts, post, scale, had_bits, order, k_cache, v_cache, pos, inv_freq, heads, kv_heads,
-                          head_dim):
+                          head_dim, key_splits=1):
     """decode_attention_rht for separate q / k / v projections: parts, post, scale, had_bits and
     order are 3-element lists (q, k, v); the three `parts` are (S, n_i) fp32 views into one
     partial-sum buffer (same number of parts and the same row stride)."""
@@ -509,13 +534,15 @@ def decode_attention_rht3(parts, post, scale, had_bits, order, k_cache, v_cache,
         raise ValueError("decode_attention_rht3: inconsistent shapes")
     dev = parts[0].device
     out = torch.empty(heads * head_dim, dtype=torch.float16, device=dev)
+    ws = _split_workspace(dev, heads, head_dim, key_splits)
     vp = lambda ts: (ctypes.c_void_p * 3)(*[t.data_ptr() if t is not None else None for t in ts])
     with torch.cuda.device(dev):
         check(lib().qtip_decode_attention_rht3(_ptr(out), vp(parts), parts[0].shape[0], parts[0].stride(0), vp(post),
                                                (ctypes.c_float * 3)(*[float(v) for v in scale]), vp(had_bits),
                                                (ctypes.c_int * 3)(*[int(v) for v in order]), _ptr(k_cache),
                                                _ptr(v_cache), _ptr(pos), _ptr(inv_freq), heads, kv_heads, head_dim,
-                                               max_len, stream_ptr(dev)), "qtip_decode_attention_rht3")
+                                               max_len, key_splits, _ptr(ws), stream_ptr(dev)),
+              "qtip_decode_attention_rht3")
     return out
 
 

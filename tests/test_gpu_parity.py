@@ -506,6 +506,63 @@ def test_decode_attention(heads, kv_heads, pos):
     assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,D,pos,splits", [(32, 32, 128, 1000, 8), (32, 32, 128, 4000, 8),
+                                                          (32, 32, 128, 4095, 16), (64, 8, 128, 4000, 4),
+                                                          (8, 8, 64, 3000, 8), (32, 32, 128, 5, 8),
+                                                          (32, 32, 128, 511, 8), (32, 32, 128, 512, 8),
+                                                          (16, 4, 128, 2047, 2)])
+def test_decode_attention_over_key_ranges(heads, kv_heads, D, pos, splits):
+    """Long contexts: the keys of a head cut into ranges (one workgroup each) and combined by a
+    second launch, against a float32 attention over the same cache (model/llama.py:866-880) and
+    against the one-workgroup form; ranges past the last key are empty (short context, many ranges)."""
+    from qtip_amd import ops
+    max_len = 4096
+    g = torch.Generator().manual_seed(pos + heads + splits)
+    qkv = torch.randn((heads + 2 * kv_heads) * D, generator=g).half().cuda()
+    kc = (torch.randn(1, kv_heads, max_len, D, generator=g) * 0.5).half().cuda()
+    vc = torch.randn(1, kv_heads, max_len, D, generator=g).half().cuda()
+    kc1, vc1 = kc.clone(), vc.clone()
+    inv_freq = (1.0 / (10000.0**(torch.arange(0, D, 2).float() / D))).cuda()
+    p = torch.tensor([pos], device="cuda")
+    one = ops.decode_attention(qkv, kc1, vc1, p, inv_freq, heads, kv_heads, D)
+    out = ops.decode_attention(qkv, kc, vc, p, inv_freq, heads, kv_heads, D, key_splits=splits)
+    assert torch.equal(kc, kc1) and torch.equal(vc, vc1)  # the same cache rows written once
+    # float32 reference on the cache as the kernel left it (row `pos` holds the rotated new key)
+    q = qkv[:heads * D].view(heads, D).float()
+    ang = pos * inv_freq
+    cos = torch.cat([ang.cos(), ang.cos()]).half().float()
+    sin = torch.cat([ang.sin(), ang.sin()]).half().float()
+    rot = torch.cat([-q[:, D // 2:], q[:, :D // 2]], dim=1)
+    qe = ((q * cos).half().float() + (rot * sin).half().float()).half().float()
+    rep = heads // kv_heads
+    kk = kc[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
+    vv = vc[0, :, :pos + 1].float().repeat_interleave(rep, dim=0)
+    sc = torch.einsum("hd,htd->ht", qe, kk) / D**0.5
+    ref = torch.einsum("ht,htd->hd", sc.softmax(-1), vv).reshape(-1)
+    assert_close(out.float().cpu().numpy(), ref.cpu().numpy(), 5e-3, 2e-3)
+    assert_close(out.float().cpu().numpy(), one.float().cpu().numpy(), 5e-3, 2e-3)
+    with pytest.raises(ValueError):
+        ops.decode_attention(qkv, kc, vc, p, inv_freq, heads, kv_heads, D, key_splits=17)
+
+
+def test_generate_switches_to_key_ranges_inside_a_run():
+    """A run that crosses ops.ATTN_SPLIT_FROM records its step again with the key-range attention
+    and keeps decoding the tokens of the eager loop; a short run stays on the one-workgroup form."""
+    from qtip_amd import ops
+    from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
+    T = ops.ATTN_SPLIT_FROM
+    assert ops.attention_key_splits(T - 1) == 1 and ops.attention_key_splits(T) == 8
+    ids = torch.randint(0, cfg.vocab, (1, T - 4), generator=torch.Generator().manual_seed(4)).cuda()
+    model = LlamaDecoder(cfg, max_cache_len=T + 64)
+    a, _, _ = generate(model, ids, 10, use_graph=True)
+    assert model.cfg.attn_key_splits == 8  # crossed inside the run
+    b, _, _ = generate(LlamaDecoder(cfg, max_cache_len=T + 64), ids, 10, use_graph=False)
+    assert a.shape == (1, 10) and torch.equal(a, b)
+    short, _, _ = generate(model, ids[:, :20], 4)
+    assert model.cfg.attn_key_splits == 1 and short.shape == (1, 4)
+
+
 @pytest.mark.parametrize("heads,kv_heads,D,S", [(32, 32, 128, 1), (64, 8, 128, 2), (8, 8, 128, 3), (16, 16, 64, 1),
                                                  (4, 2, 128, 2), (4, 2, 64, 5), (56, 8, 128, 1)])
 def test_decode_attention_with_output_transform_in_prologue(heads, kv_heads, D, S):
