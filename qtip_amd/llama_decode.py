@@ -240,7 +240,8 @@ class DecoderLayer(nn.Module):
             if ok:
                 f = self._fused_linears()
                 cfg = self.cfg
-                ok = not any(l.dense for l in f.values()) and cfg.hidden in ops.RHT_IN_MATVEC_SIZES
+                ok = (not any(l.dense or l.shard_in or l.shard_out for l in f.values())
+                      and cfg.hidden in ops.RHT_IN_MATVEC_SIZES)
                 if ok:
                     q, k, v, g, u, o, d = (f[n] for n in ('q_proj', 'k_proj', 'v_proj', 'gate_proj', 'up_proj', 'o',
                                                           'down'))
@@ -263,7 +264,7 @@ class DecoderLayer(nn.Module):
             if ok:
                 f = self._fused_linears()
                 cfg = self.cfg
-                ok = not any(l.dense for l in f.values())
+                ok = not any(l.dense or l.shard_in or l.shard_out for l in f.values())
                 if ok:
                     q, k, v, g, u = (f[n] for n in ('q_proj', 'k_proj', 'v_proj', 'gate_proj', 'up_proj'))
                     ok = (q.K == k.K == v.K and g.K == u.K and g.m == u.m and g.Kr == u.Kr
@@ -374,12 +375,24 @@ class _FusedLinear:
     def __init__(self, lin):
         self.lin = lin
         self.dense = isinstance(lin, nn.Linear)
+        self.shards, self.shard_in, self.shard_out = 1, False, False
         if self.dense:
             return
-        if not lin.has_kernel or int(lin.rcp) != 0:
-            raise NotImplementedError("fused decode needs kernel-packed HYB layers with rcp == 0")
+        if not lin.has_kernel:
+            raise NotImplementedError("fused decode needs kernel-packed HYB layers")
         dev = lin.trellis.device
         self.n, self.m, self.K = lin.in_features, lin.out_features, lin.K
+        # per-shard transforms (lib/codebook/bitshift.py:437-441,465-469): rcp 1 applies the input
+        # transform to each of the tp_rank slices of the input, rcp 2 the output transform to each
+        # slice of the output.  Such a side keeps its transform as a launch of its own (tp_rank rows
+        # of a smaller transform) and takes no part in the launches that fold transforms into their
+        # neighbours.
+        rcp = int(lin.rcp)
+        self.shards = int(lin.tp_rank) if rcp in (1, 2) else 1
+        self.shard_in = rcp == 1 and self.shards > 1
+        self.shard_out = rcp == 2 and self.shards > 1
+        if (self.shard_in and self.n % self.shards) or (self.shard_out and self.m % self.shards):
+            raise NotImplementedError("tp_rank does not divide the sharded side")
         self.trellis = lin.trellis.reshape(-1)
         self.tlut = lin.tlut.data.reshape(-1).contiguous()
         self.SU, self.SV = lin.SU, lin.SV
@@ -398,6 +411,16 @@ class _FusedLinear:
         return y if residual is None else residual + y
 
     def transform_in(self, x, pre_mode=ops.PRE_NONE, norm_weight=None, eps=0.0):
+        if self.shard_in:
+            if pre_mode == ops.PRE_RMSNORM:
+                x = ops.rmsnorm(x.reshape(-1), norm_weight, eps)
+            elif pre_mode == ops.PRE_SILU_MUL:
+                gate, up = x.reshape(-1).split(x.numel() // 2)
+                x = F.silu(gate) * up
+            ns = self.n // self.shards
+            xf = (x.reshape(-1).float() * self.SU).reshape(self.shards, ns)
+            return ops.rht(xf, order=self.Kl, had_bits=self.bl, scale=(ns**-0.5) / 32.0,
+                           out_dtype=torch.float16).reshape(1, self.n)
         return ops.rht(x, order=self.Kl, had_bits=self.bl, pre=self.SU, scale=(self.n**-0.5) / 32.0,
                        out_dtype=torch.float16, pre_mode=pre_mode, norm_weight=norm_weight, eps=eps)
 
@@ -409,12 +432,20 @@ class _FusedLinear:
         """matvec(transform_in(x)) for a plain input; one launch when the transform is a power of
         two the matvec kernel computes in its prologue."""
         if (self.Kl == 1 and self.n in ops.RHT_IN_MATVEC_SIZES and x.dtype == torch.float16
-                and self.SU.dtype == torch.float16):
+                and self.SU.dtype == torch.float16 and not self.shard_in):
             return ops.decompress_matvec_parts_rht(self.trellis, x.reshape(-1), self.SU, (self.n**-0.5) / 32.0,
                                                    self.tlut, self.m, self.n, self.K).unsqueeze(1)
         return self.matvec(self.transform_in(x))
 
     def transform_out(self, parts, residual=None):
+        if self.shard_out:
+            y = parts.reshape(parts.shape[0], self.m)
+            y = y.sum(0) if y.shape[0] > 1 else y[0]
+            ms = self.m // self.shards
+            yt = ops.rht(y.reshape(self.shards, ms), order=self.Kr, had_bits=self.br, scale=ms**-0.5,
+                         out_dtype=torch.float32).reshape(1, self.m)
+            out = (yt * (self.SV * 32.0)).to(torch.float16)
+            return out if residual is None else residual + out
         return ops.rht(parts if parts.shape[0] > 1 else parts.reshape(1, self.m), order=self.Kr, had_bits=self.br,
                        post=self.SV, scale=(self.m**-0.5) * 32.0, out_dtype=torch.float16, in_parts=parts.shape[0],
                        residual=residual)
@@ -422,7 +453,7 @@ class _FusedLinear:
     def transform_out_silu(self, parts):
         """Output transform of a fused up/gate projection; where one launch can pair the halves it
         also applies SiLU(gate) * up and returns (1, m / 2) instead of (1, m)."""
-        if ops.rht_silu_pair_ok(self.m, self.Kr, False):
+        if not self.shard_out and ops.rht_silu_pair_ok(self.m, self.Kr, False):
             return ops.rht_silu_pair(parts.reshape(parts.shape[0], self.m), self.SV, order=self.Kr, had_bits=self.br,
                                      scale=(self.m**-0.5) * 32.0).reshape(1, -1)
         return self.transform_out(parts)
@@ -431,14 +462,14 @@ class _FusedLinear:
         """The output transform can run in the attention kernel's prologue (head-sized slices of a
         table-order x power-of-two transform)."""
         p2 = self.m // self.Kr
-        return (not self.dense and head_dim in (64, 128) and p2 >= head_dim and p2 & (p2 - 1) == 0
-                and self.m <= 16384)
+        return (not self.dense and not self.shard_out and head_dim in (64, 128) and p2 >= head_dim
+                and p2 & (p2 - 1) == 0 and self.m <= 16384)
 
     def can_chain_into(self, nxt):
         """This layer's output transform and `nxt`'s input transform are plain power-of-two
         transforms of one hidden-size vector: one launch does both plus residual and RMSNorm."""
         return (not self.dense and not nxt.dense and self.Kr == 1 and nxt.Kl == 1 and self.m == nxt.n
-                and self.m in (2048, 4096, 8192))
+                and self.m in (2048, 4096, 8192) and not self.shard_out and not nxt.shard_in)
 
     def chain(self, parts, residual, nxt, norm_weight, eps):
         """(x_new, xt): transform_out(parts) + residual, then nxt.transform_in(RMSNorm(x_new))."""
@@ -519,9 +550,9 @@ class LlamaDecoder(nn.Module):
         return (x @ self.lm_head.T).float()
 
     def supports_fused_decode(self):
-        """False when a layer needs what the fused decode step does not cover (per-shard
-        transforms, rcp != 0, a layer that is not kernel-packed, or a key / value cache longer than
-        the attention kernel's FUSED_MAX_CACHE_LEN slots): generate() then decodes module by module."""
+        """False when a layer needs what the fused decode step does not cover (a layer that is not
+        kernel-packed, or a key / value cache longer than the attention kernel's
+        FUSED_MAX_CACHE_LEN slots): generate() then decodes module by module."""
         if self.max_cache_len > FUSED_MAX_CACHE_LEN:
             return False
         try:

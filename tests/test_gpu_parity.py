@@ -900,19 +900,67 @@ def test_synthetic_model_tables_leave_no_rank_one_part():
     assert float(lg.float().abs().max()) < 100
 
 
-def test_generate_falls_back_for_per_shard_transforms():
-    """A model quantised with per-shard transforms (rcp != 0) is outside the fused decode step:
-    generate() decodes it module by module instead of failing."""
+@pytest.mark.parametrize("fused", [True, False])
+def test_fused_decode_with_per_shard_transforms(fused):
+    """Layers quantised with per-shard transforms (rcp 1: input side, rcp 2: output side, tp_rank
+    slices; lib/codebook/bitshift.py:437-441,465-469) run inside the fused decode step: their sharded
+    side keeps its transform as a launch of tp_rank rows, everything else stays folded.  Checked
+    against the module-by-module forward (whose layer forward is held to the oracle for rcp 1 / 2),
+    on both projection layouts, eagerly and through generate()'s recorded graph."""
     from qtip_amd.llama_decode import LlamaConfig, LlamaDecoder, generate
-    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=2, ffn=172 * 16, vocab=512)
-    model = LlamaDecoder(cfg, max_cache_len=64)
-    ids = torch.randint(0, cfg.vocab, (1, 5), generator=torch.Generator().manual_seed(2)).cuda()
-    assert LlamaDecoder(cfg, max_cache_len=64).supports_fused_decode()
-    model.layers[1].down.rcp.fill_(1)
-    model.layers[1].down.tp_rank.fill_(1)  # one shard: the same transform, through the general path
-    assert not model.supports_fused_decode()
-    out, _, _ = generate(model, ids, 5, use_graph=True, fused=True)
-    assert out.shape == (1, 5)
+    cfg = LlamaConfig(hidden=1024, heads=8, kv_heads=8, layers=3, ffn=172 * 16, vocab=512)
+    model = LlamaDecoder(cfg, max_cache_len=64, fused=fused)
+
+    def shard(lin, rcp, tp):
+        if isinstance(lin.rcp, torch.Tensor):  # plain ints after the module's first forward
+            lin.rcp.fill_(rcp)
+            lin.tp_rank.fill_(tp)
+        else:
+            lin.rcp, lin.tp_rank = rcp, tp
+
+    l0, l1, l2 = model.layers
+    shard(l0.o, 1, 8)
+    shard(l0.down, 2, 4)
+    if fused:
+        shard(l1.qkv, 2, 8)       # 3072 outputs: 8 slices of 384 = 12 x 32
+        shard(l1.up_gate, 1, 4)
+        shard(l2.up_gate, 2, 8)   # 5504 outputs: 8 slices of 688 = 172 x 4
+        shard(l2.qkv, 1, 2)
+    else:
+        shard(l1.k_proj, 2, 8)
+        shard(l1.gate_proj, 1, 4)
+        shard(l2.up_proj, 2, 8)   # 2752 outputs: 8 slices of 344 = 172 x 2
+        shard(l2.q_proj, 1, 2)
+    shard(l2.down, 1, 4)          # 2752 inputs: 4 slices of 688
+    assert model.supports_fused_decode()
+    ids = torch.randint(0, cfg.vocab, (1, 9), generator=torch.Generator().manual_seed(0)).cuda()
+    with torch.no_grad():
+        lg = model(ids, torch.arange(9, device="cuda"))
+        tok = lg[:, -1].argmax(-1, keepdim=True)
+        pos = torch.tensor([9], device="cuda")
+        a = model(tok, pos)
+        kc = [c.clone() for c in model.k_cache]
+        b = model.decode_fused(tok, pos)
+    assert bool(torch.isfinite(b).all())
+    assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+    for c0, c1 in zip(kc, model.k_cache):
+        assert torch.allclose(c0.float(), c1.float(), atol=2e-2)
+    # a sharded side really changes the result: the same weights read as rcp 0 decode differently
+    shard(l0.o, 0, 8)
+    for name in ("_fused", "_grouped", "_grouped_plain"):
+        l0.__dict__.pop(name, None)
+    with torch.no_grad():
+        c = model.decode_fused(tok, pos)
+    assert float((c - b).abs().max()) > 1e-2
+    shard(l0.o, 1, 8)
+    for name in ("_fused", "_grouped", "_grouped_plain"):
+        l0.__dict__.pop(name, None)
+    out_g, _, _ = generate(model, ids, 6, use_graph=True, fused=True)
+    out_e, _, _ = generate(model, ids, 6, use_graph=False, fused=True)
+    out_m, _, _ = generate(model, ids, 6, use_graph=False, fused=False)
+    assert torch.equal(out_g, out_e)
+    assert out_g.shape == (1, 6) and out_m.shape == (1, 6)
+    assert int((out_g == out_m).sum()) >= 5  # greedy picks may part on a near-tie late in the run
 
 
 def test_sample_pick_draws_from_the_reference_distribution():
