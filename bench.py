@@ -385,8 +385,21 @@ def main():
             gr = capture(lambda: [fn() for _ in range(4)])
             ceil[name + "_GBps"] = round(moved / (timed(gr, 3, args.settle_ms / 3) / 4) / 1e9, 1)
             del gr
-        result["measured_ceilings"] = ceil
         del src, dst
+        # issue rates of the instructions the 2-bit decode consists of, and its loop without memory:
+        # ns one wave-instruction (one wave-load) occupies a SIMD with 4 waves per SIMD, as in the matvec
+        issue = {}
+        iters = 2000
+        for name in ops.PROBE_KINDS:
+            gr = capture(lambda: ops.probe_issue(name, iters, tlut))
+            t = timed(gr, 3, args.settle_ms / 6)
+            per = iters * 4 * (1 if name.startswith("decode_loop") else ops.PROBE_OPS_PER_ITER)
+            issue[name] = round(t * 1e9 / per, 2 if per > iters * 4 else 1)
+            del gr
+        ceil["issue_ns_per_wave_instruction_and_simd"] = {k: v for k, v in issue.items() if not k.startswith("decode_loop")}
+        ceil["decode_loop_ns_per_wave_load_and_simd"] = {
+            "loop_without_memory": issue["decode_loop"], "vector_alu_part_alone": issue["decode_loop_valu"]}
+        result["measured_ceilings"] = ceil
 
     if "decode" in extras:
         # packed -> dense fp16 weights (the reference's decode_compressed); bound by the dense write

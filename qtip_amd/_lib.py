@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("QTIP_HIP_LIBRARY") or os.path.join(_HERE, "libqtip_hi
 
 QTIP_F16 = 0
 QTIP_F32 = 1
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 _lib = None
 
@@ -79,6 +79,7 @@ _SIGNATURES = {
     "qtip_sample_pick": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_uint] +
                          [ctypes.c_void_p] * 4 + [ctypes.c_long, ctypes.c_long, ctypes.c_void_p]),
     "qtip_probe_stream_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "qtip_probe_issue": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "qtip_repack": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "qtip_unpack_trellis": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_long] + [ctypes.c_int] * 3 +
                             [ctypes.c_void_p]),

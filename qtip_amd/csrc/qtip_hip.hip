@@ -1285,6 +1285,10 @@ __global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict_
 constexpr size_t kScratchFloats = 64 * 1024;  // 256 KiB
 static __device__ __align__(256) float scratch[kScratchFloats];
 
+}  // namespace
+#include "qtip_probe.h"
+namespace {
+
 template <typename F>
 hipError_t allow_lds(F* fn, size_t bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
@@ -1327,6 +1331,9 @@ hipError_t allow_lds_all() {
   QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
   QTIP_ALLOW((gemm4_kernel<1>), kGemm4Lds)
   QTIP_ALLOW((gemm4_kernel<2>), kGemm4Lds)
+  QTIP_ALLOW((issue_probe_kernel<kProbeDsRead>), kProbeLds)
+  QTIP_ALLOW((loop_probe_kernel<0>), kProbeLds)
+  QTIP_ALLOW((loop_probe_kernel<1>), kProbeLds)
 #undef QTIP_ALLOW
   return hipSuccess;
 }
@@ -1451,7 +1458,7 @@ int choose_split(int m, int k, int bits, int cus, bool summed) {
 
 extern "C" {
 
-int qtip_abi_version(void) { return 19; }
+int qtip_abi_version(void) { return 20; }
 
 int qtip_init(void) { return (int)device_state().status; }
 
@@ -1922,5 +1929,37 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   }
   return QTIP_OK;
 }
+
+int qtip_probe_issue(int kind, int iters, const void* tlut, void* sink_u32, void* stream) {
+  if (!tlut || !sink_u32) return QTIP_E_NULL;
+  if (iters < 1 || iters > (1 << 20)) return QTIP_E_SHAPE;
+  if (const int rc = ready_code(stream)) return rc;
+  const DeviceInfo di = device_info();
+  hipStream_t st = (hipStream_t)stream;
+  const uint32_t* tl = (const uint32_t*)tlut;
+  uint32_t* sink = (uint32_t*)sink_u32;
+  switch (kind) {
+#define QTIP_PROBE(KIND, LDS) \
+  case KIND: issue_probe_kernel<KIND><<<di.cus, 1024, LDS, st>>>(iters, tl, sink); break;
+    QTIP_PROBE(kProbeAnd, 0)
+    QTIP_PROBE(kProbeAddU32, 0)
+    QTIP_PROBE(kProbeLshrImm, 0)
+    QTIP_PROBE(kProbeLshlImm, 0)
+    QTIP_PROBE(kProbePkMad, 0)
+    QTIP_PROBE(kProbeMadU32U16, 0)
+    QTIP_PROBE(kProbePerm, 0)
+    QTIP_PROBE(kProbePkLshr, 0)
+    QTIP_PROBE(kProbeMovDpp, 0)
+    QTIP_PROBE(kProbeDot2c, 0)
+    QTIP_PROBE(kProbeDsRead, kProbeLds)
+    QTIP_PROBE(kProbeMfma, 0)
+#undef QTIP_PROBE
+    case kProbeLoop: loop_probe_kernel<0><<<di.cus, 1024, kProbeLds, st>>>(iters, tl, sink); break;
+    case kProbeLoopValu: loop_probe_kernel<1><<<di.cus, 1024, kProbeLds, st>>>(iters, tl, sink); break;
+    default: return QTIP_E_SHAPE;
+  }
+  return (int)hipGetLastError();
+}
+
 
 }  // extern "C"
