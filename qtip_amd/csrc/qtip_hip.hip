@@ -5,6 +5,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "../../include/qtip_hip.h"
 #include "qtip_device.h"
@@ -151,7 +152,12 @@ constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a w
 // product whenever lanes i and j read the same columns, i.e. i % 2 == j % 2.  Lane (g, a) keeps
 // D[4g + r][a] in element r, so element a % 2 of the accumulator is the lane's row sum over all
 // four blocks of the wave-load (the cross-block reduction happens inside the MFMA).
-template <int K>
+//
+// RH = 0 / 1 decodes only the states of row half rh = RH (rows 8*RH .. 8*RH + 7 of either tile
+// row half): the registers P[i] with i % 2 == RH at every bit width, half the hashes, lookups and
+// MFMAs and - the extraction of the others being dead code - about half the vector work.  The
+// accumulators of the other row half stay untouched.
+template <int K, int RH = -1>
 __device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u32x2 xv[4],
                                                        uint32_t slot4, float4_t acc[4]) {
   uint32_t P[16], W[32];
@@ -159,6 +165,7 @@ __device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
+    if (RH >= 0 && (i & 1) != RH) continue;
     const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
     W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
     W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
@@ -171,6 +178,7 @@ __device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u
     for (int mh = 0; mh < 2; ++mh)
 #pragma unroll
       for (int rh = 0; rh < 2; ++rh) {
+        if (RH >= 0 && rh != RH) continue;
         const int tt = 2 * kh + mh;
         const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
                           W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
@@ -396,7 +404,13 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 // x is staged in two halves, the second replacing the first in the middle of the unit (two more
 // barriers per launch instead of x travelling through vector loads with every wave-load, which
 // made the 28672-wide matrices 15-20 % slower).
-template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false, bool GROUP = false>
+// HALF: the row blocks that do not fill a last round of whole units (at most half a round of
+// them) are cut by row half instead: workgroup w < upw_r takes the rows with rh = w % 2 of row
+// block upw_q * rb_step + w / 2 after its upw_q whole units.  Such a half unit reads the block's
+// whole stream but decodes half of its states (about 0.55 of a unit's time), and its rows are
+// complete sums, so nothing has to be combined across workgroups: 320 row blocks on 256
+// workgroups take 1.55 units of time instead of 2, 128 row blocks 0.55 instead of 1.
+template <int K, int DEPTH, bool XLDS, int XFORM = 0, bool XHALF = false, bool GROUP = false, bool HALF = false>
 __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     float* __restrict__ dst_, const uint8_t* __restrict__ packed_, const uint16_t* __restrict__ x_,
     const uint32_t* __restrict__ tlut_, int m_, int k, int wl_per, int upw_q_, int upw_r_,
@@ -417,6 +431,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const int upw_q = GROUP ? pick3(grp.upw_q, gi) : upw_q_;
   const int upw_r = GROUP ? pick3(grp.upw_r, gi) : upw_r_;
   static_assert(!XHALF || (XLDS && !XFORM), "two-half staging is a form of the plain staged x");
+  static_assert(!HALF || (XLDS && !XFORM && !XHALF && !GROUP), "half units exist for the plain form with x in LDS");
   constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
@@ -445,8 +460,14 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const int wl1 = wl0 + wl_per < nwl ? wl0 + wl_per : nwl;
   const int wl1f = wl1 < nfull ? wl1 : nfull;           // end of the full wave-loads
   const int npw = (wl_per + kWaves - 1) / kWaves;       // items per wave and unit (padded)
-  const int upw = upw_q + (rb0 < upw_r ? 1 : 0);  // units of this workgroup: ceil((nrb - rb0) / rb_step), quotient and remainder from the host
-  const int T = upw * npw;
+  // whole units of this workgroup: ceil((nrb - rb0) / rb_step), quotient and remainder from the host;
+  // with HALF the remainder counts half units instead
+  const int upw = HALF ? upw_q : upw_q + (rb0 < upw_r ? 1 : 0);
+  const int T_full = upw * npw;
+  const bool has_half = HALF && rb0 < upw_r;
+  const int half_rh = rb0 & 1;
+  const int half_rb = upw_q * rb_step + (rb0 >> 1);
+  const int T = T_full + (has_half ? npw : 0);
   const int w_first = wl0 + wave;
   const int nvj = w_first < wl1f ? (wl1f - w_first + kWaves - 1) / kWaves : 0;  // real items per unit
   const bool tail_wave = wl1 > nfull && ((nfull - wl0) % kWaves) == wave;
@@ -459,7 +480,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 
   // load cursor: unit l_i (row block l_rb), item l_j
   int l_j = 0, l_t = 0;
-  uint32_t l_rboff = (uint32_t)rb0 * rb_bytes;
+  uint32_t l_rboff = (uint32_t)((HALF && upw == 0) ? half_rb : rb0) * rb_bytes;
   const uint32_t rb_step_bytes = (uint32_t)rb_step * rb_bytes;
   LaneData<K> buf[DEPTH];
   u32x2 xbuf[XLDS ? 1 : DEPTH][4];
@@ -476,7 +497,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     ++l_t;
     if (++l_j == npw) {
       l_j = 0;
-      l_rboff += rb_step_bytes;
+      l_rboff = (HALF && l_t == T_full) ? (uint32_t)half_rb * rb_bytes : l_rboff + rb_step_bytes;
     }
   };
   // Prologue loads in the order they are needed: the table words and x first, then the first
@@ -494,9 +515,11 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const uint32_t* tp = tlut + it * 128 + wave * 8;
-    uint32_t sw[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) sw[j] = tp[j];
+    // one 32-byte scalar load (the table needs dword alignment only).  Loaded word by word, the
+    // compiler may fold the first select below into a per-lane load of tp[lane >> 3], and the wait
+    // for that vector load also waits for the stream loads requested before it.
+    typedef uint32_t u32x8_dw __attribute__((ext_vector_type(8), aligned(4)));
+    const u32x8_dw sw = *reinterpret_cast<const u32x8_dw*>(tp);
     uint32_t v = sw[0];
 #pragma unroll
     for (int j = 1; j < 8; ++j) v = ((lane >> 3) == j) ? sw[j] : v;
@@ -596,13 +619,18 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   float4_t acc[4];  // [2*mh + rh]: rows 16*mh + 8*rh + a/2 of the unit's 32-row block
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-  auto accumulate = [&](const LaneData<K>& ld, const u32x2 xv[4]) {
-    matvec_accumulate<K>(ld, xv, slot4, acc);
-  };
-  int parity = 0, c_j = 0, c_rb = rb0;
+  int parity = 0, c_j = 0, c_rb = (HALF && upw == 0) ? half_rb : rb0;
   int c_jbase = 0;  // first item of the staging that is in LDS
   int prio_phase = wave >> 2;  // waves w, w + 4, w + 8, w + 12 share a SIMD
-  for (int t = 0; t < T; t += DEPTH) {
+  // items [t0, t1) of the workgroup's item sequence, decoding all states (RH = -1) or one row half.
+  // Whole and half units run in loops of their own: with both forms behind a branch in one loop
+  // body the compiler loses track of the loads in flight and waits for all of them at every item.
+  auto run = [&](auto rh_tag, const int t0, const int t1) {
+  constexpr int RH = decltype(rh_tag)::value;
+  auto accumulate = [&](const LaneData<K>& ld, const u32x2 xv[4]) {
+    matvec_accumulate<K, RH>(ld, xv, slot4, acc);
+  };
+  for (int t = t0; t < t1; t += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       // The hardware serves the waves of a SIMD oldest first, so the oldest finishes its share of a
@@ -614,7 +642,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
         case 2: __builtin_amdgcn_s_setprio(2); break;
         default: __builtin_amdgcn_s_setprio(3); break;
       }
-      if (t + d < T) {
+      if (t + d < t1) {
         if (c_j < nvj) {
           if constexpr (XLDS) {
             typedef __attribute__((address_space(3))) const u32x2 lds_u32x2_t;
@@ -631,10 +659,10 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       // the stage's registers are refilled only after their last use, so the
       // refill reuses them in place (no copies, no wait on the new load)
       issue(d);
-      if (t + d < T) ++c_j;
+      if (t + d < t1) ++c_j;
       if constexpr (XHALF) {
         // middle of the (only) unit: every wave has read its last x of the first half
-        if (t + d < T && c_j == jh && jh < npw) {
+        if (t + d < t1 && c_j == jh && jh < npw) {
           __syncthreads();
           const int xbytes2 = (wl1 - wl0 - wlx) * 256;
 #pragma unroll
@@ -646,7 +674,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           c_jbase = jh;
         }
       }
-      if (t + d < T && c_j == npw) {
+      if (t + d < t1 && c_j == npw) {
         // ---- end of a unit: ragged tail, reductions, store
         // k/32 not a multiple of 4: one wave takes the partial wave-load.  Every lane takes part
         // in an MFMA, so the lanes of the missing blocks read x = 0 (the descriptor of x ends
@@ -670,7 +698,8 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
           if (g == 0 && (a & 1) == 0) pp[wave * 32 + (i >> 1) * 16 + (i & 1) * 8 + (a >> 1)] = v;
         }
         __syncthreads();
-        if (tid < 32) {
+        // (a half unit owns the rows 16*mh + 8*rh + 0..7 of its rh only)
+        if (tid < 32 && (RH < 0 || ((tid >> 3) & 1) == RH)) {
           float sum = 0.f;
 #pragma unroll
           for (int w = 0; w < kWaves; ++w) sum += pp[w * 32 + tid];
@@ -678,8 +707,16 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
         }
         parity ^= 1;  // the other buffer is free: its readers passed the barrier above
         c_j = 0;
-        c_rb += rb_step;
+        c_rb = (HALF && t + d + 1 == T_full) ? half_rb : c_rb + rb_step;
       }
+    }
+  }
+  };
+  run(std::integral_constant<int, -1>{}, 0, T_full);
+  if constexpr (HALF) {
+    if (has_half) {
+      if (half_rh) run(std::integral_constant<int, 1>{}, T_full, T);
+      else run(std::integral_constant<int, 0>{}, T_full, T);
     }
   }
 }
@@ -1308,6 +1345,7 @@ hipError_t allow_lds_all() {
   QTIP_ALLOW((matvec_kernel<2, 2, true>), kMatvecLds + kMatvecXBytes)
   QTIP_ALLOW((matvec_kernel<3, 2, true>), kMatvecLds + kMatvecXBytes)
   QTIP_ALLOW((matvec_kernel<4, 2, true>), kMatvecLds + kMatvecXBytes)
+  QTIP_ALLOW((matvec_kernel<2, 2, true, 0, false, false, true>), kMatvecLds + kMatvecXBytes)
   QTIP_ALLOW((matvec_kernel<2, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
   QTIP_ALLOW((matvec_kernel<3, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
   QTIP_ALLOW((matvec_kernel<4, 2, true, 0, false, true>), kMatvecLds + kMatvecXBytes)
@@ -1553,6 +1591,25 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
     return (int)hipGetLastError();
   }
   const size_t xbytes = (size_t)wl_per * 256;
+  // row blocks left over by the rounds of whole units, when they fill at most half a round of the
+  // full grid: each is cut into its two row halves (see HALF at the kernel).  The half units follow
+  // the whole ones in the same two-stage load pipeline, so the whole units must end on an even
+  // item.  Measured: 10240x8192 11.1 -> 9.9 us, 12288x4096 7.15 -> 6.75 us at 2 bits.  Not used
+  // where it measured slower: without a round of whole units before them (twice the workgroups
+  // and twice the stream for matrices that are latency-bound anyway: 4096x4096 4.8 -> 5.3 us) and
+  // at 3 and 4 bits (the doubled stream of the left-over blocks costs what the halved decode saves).
+  const int full_range = di.cus / S;
+  const int left = full_range > 0 ? (m >> 5) % full_range : 0;
+  const int whole = full_range > 0 ? (m >> 5) / full_range : 0;
+  const bool even_items = (((wl_per + kWaves - 1) / kWaves) & 1) == 0;
+#ifndef QTIP_NO_HALF_UNITS
+  if (bits == 2 && xbytes <= kMatvecXBytes && left > 0 && 2 * left <= full_range && whole >= 1 && even_items) {
+    const dim3 gh((unsigned)S, (unsigned)full_range);
+    matvec_kernel<2, 2, true, 0, false, false, true><<<gh, kThreads, kMatvecLds + xbytes, st>>>(
+        dst, p, xx, t, m, k, wl_per, whole, 2 * left);
+    return (int)hipGetLastError();
+  }
+#endif
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {

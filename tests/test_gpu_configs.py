@@ -43,6 +43,46 @@ def assert_close(got, ref, max_rel=MAX_REL, mean_rel=MEAN_REL):
     assert mx <= max_rel and mn <= mean_rel, (mx, mn)
 
 
+# (m, k, partial vectors): row blocks = whole rounds of the 256 / nparts workgroups of a k range plus
+# a left-over of at most half a round, and an even number of wave-loads per wave and unit - the
+# left-over row blocks are then cut into their two row halves (rows 8*rh .. 8*rh+7 of either tile
+# row half) instead of running as a sparse last round
+HALF_UNIT_CASES = [(8192 + 32 * 5, 4096, 1), (8192 + 32 * 128, 8192, 1), (2 * 8192 + 32 * 77, 4096, 1),
+                   (10240, 4000, 1),             # ragged k: 31 full wave-loads per row block and a quarter one
+                   (4096 + 32 * 40, 8192, 2),    # two k ranges of 128 workgroups each
+                   (8192 + 32 * 129, 4096, 1)]   # one block too many for halves: a plain last round
+
+
+@pytest.mark.parametrize("m,k,nparts", HALF_UNIT_CASES)
+def test_matvec_with_left_over_row_blocks_cut_by_row_half(m, k, nparts):
+    """2-bit matvec on row-block counts that leave a partial last round: every row against the
+    oracle (a half unit writes 16 of its block's 32 rows, its sibling the other 16), bitwise
+    equal repeats, and the partial vectors of a k split."""
+    from qtip_amd import ops
+    K = 2
+    L = make_layer(m, k, K, seed=m + k + nparts)
+    pk, tl = dev(L["packed"]), dev(L["tlut"])
+    x = L["x"].reshape(-1)
+    ref = c_oracle.matvec(L["packed"], x, L["tlut"], m, k, K)
+    if nparts == 1:
+        out = torch.full((m,), float("nan"), device="cuda")
+        ops.decompress_matvec(pk, dev(x), tl, m, k, K, out=out, split_k=False)
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()  # every row was written by exactly the unit that owns it
+        assert_close(got, ref)
+        again = ops.decompress_matvec(pk, dev(x), tl, m, k, K, split_k=False)
+        assert torch.equal(again, out)
+    else:
+        parts = ops.decompress_matvec_parts(pk, dev(x), tl, m, k, K, nparts=nparts)
+        assert parts.shape == (nparts, m) and bool(torch.isfinite(parts).all())
+        assert_close(parts.double().sum(0).cpu().numpy(), ref)
+        # the first k range alone: the oracle on the first half of the columns
+        half = np.zeros_like(x)
+        cols = (((k // 32 + 3) // 4 + nparts - 1) // nparts) * 128
+        half[:cols] = x[:cols]
+        assert_close(parts[0].cpu().numpy(), c_oracle.matvec(L["packed"], half, L["tlut"], m, k, K))
+
+
 @pytest.mark.parametrize("m,k,K", MATVEC_CASES)
 def test_matrix_at_full_size(m, k, K):
     """decode bit-exact; matvec with and without the k split, as partial vectors, through the
