@@ -1365,8 +1365,6 @@ hipError_t allow_lds_all() {
   QTIP_ALLOW((gemm_kernel<2, 2, 4, 8>), kGemmLds)
   QTIP_ALLOW((gemm_kernel<3, 1, 2, 16>), kGemmLds)
   QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
-  QTIP_ALLOW((gemm_kernel<4, 1, 2, 16>), kGemmLds)
-  QTIP_ALLOW((gemm_kernel<4, 2, 2, 8>), kGemmLds)
   QTIP_ALLOW((gemm4_kernel<1>), kGemm4Lds)
   QTIP_ALLOW((gemm4_kernel<2>), kGemm4Lds)
   QTIP_ALLOW((issue_probe_kernel<kProbeDsRead>), kProbeLds)
@@ -1602,14 +1600,12 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   const int left = full_range > 0 ? (m >> 5) % full_range : 0;
   const int whole = full_range > 0 ? (m >> 5) / full_range : 0;
   const bool even_items = (((wl_per + kWaves - 1) / kWaves) & 1) == 0;
-#ifndef QTIP_NO_HALF_UNITS
   if (bits == 2 && xbytes <= kMatvecXBytes && left > 0 && 2 * left <= full_range && whole >= 1 && even_items) {
     const dim3 gh((unsigned)S, (unsigned)full_range);
     matvec_kernel<2, 2, true, 0, false, false, true><<<gh, kThreads, kMatvecLds + xbytes, st>>>(
         dst, p, xx, t, m, k, wl_per, whole, 2 * left);
     return (int)hipGetLastError();
   }
-#endif
   if (xbytes <= kMatvecXBytes) {
     const size_t lds = kMatvecLds + xbytes;
     switch (bits) {
@@ -1934,11 +1930,7 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   // up to 16 rows run on the 16-wave workgroup (4 wave-loads per stage)
   for (int b0 = 0; b0 < batch; b0 += 32) {
     const int nb = batch - b0 < 32 ? batch - b0 : 32;
-#ifndef QTIP_NO_GEMM4
     const bool rowsplit = bits == 4;  // the 4-bit kernel without duplicated products, 16 waves for every batch
-#else
-    const bool rowsplit = false;
-#endif
     const int KS = (rowsplit || nb <= 16) ? 4 : 2;
     int Sp = S;
     int wl_per = (nwl + Sp - 1) / Sp;
@@ -1954,7 +1946,7 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
     const int rnd = Sp > 1 ? 0 : round_f16;
     const uint16_t* xx = (const uint16_t*)x_f16 + (size_t)b0 * k;
 #define QTIP_GEMM(KB, NBT, WV)                                                                          \
-  gemm_kernel<KB, NBT, (KB == 2 ? 4 : KB == 3 ? (WV == 16 ? 2 : 4) : 2), WV><<<g2, WV * 64, kGemmLds, st>>>( \
+  gemm_kernel<KB, NBT, (KB == 2 ? 4 : (WV == 16 ? 2 : 4)), WV><<<g2, WV * 64, kGemmLds, st>>>( \
       d, p, xx, t, m, k, nb, rnd, wl_per, ngroups / per_range, ngroups % per_range)
 #define QTIP_GEMM_K(KB)               \
   if (nb <= 16) QTIP_GEMM(KB, 1, 16); \
@@ -1967,11 +1959,7 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
         gemm4_kernel<2><<<g2, kThreads, kGemm4Lds, st>>>(d, p, xx, t, m, k, nb, rnd, wl_per, ngroups / per_range,
                                                          ngroups % per_range);
     } else {
-      switch (bits) {
-        case 2: QTIP_GEMM_K(2) break;
-        case 3: QTIP_GEMM_K(3) break;
-        default: QTIP_GEMM_K(4) break;
-      }
+      if (bits == 2) { QTIP_GEMM_K(2) } else { QTIP_GEMM_K(3) }
     }
 #undef QTIP_GEMM_K
 #undef QTIP_GEMM
