@@ -1,6 +1,6 @@
 """GPU: the benchmark configurations at their full size against the CPU oracle.
 
-Every matrix shape of the Llama-2-7B set (2, 3 and 4 bits), of the Llama-2-70B set (2 bits) and
+Every matrix shape of the Llama-2-7B set and of the Llama-2-70B set (2, 3 and 4 bits) and
 of the 4-bit batched product runs here at its real size, the sizes the reference's own
 functional test uses (qtip-kernels/test_decompress_matvec.py:9-38, 275-301): these are the
 shapes with several work units per workgroup, uneven unit counts (320 or 1792 row blocks on
@@ -24,7 +24,8 @@ MEAN_REL = 1e-3
 
 SET_7B = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]
 SET_70B = [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]
-MATVEC_CASES = [(m, k, K) for K in (2, 3, 4) for (m, k) in SET_7B] + [(m, k, 2) for (m, k) in SET_70B]
+# (the benchmark line also reports the 70B set at 3 and 4 bits, so those run here as well)
+MATVEC_CASES = [(m, k, K) for K in (2, 3, 4) for (m, k) in SET_7B] + [(m, k, K) for K in (2, 3, 4) for (m, k) in SET_70B]
 
 
 def dev(a):
