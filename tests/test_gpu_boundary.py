@@ -92,6 +92,41 @@ def test_workspace_growth_keeps_the_buffer_a_recorded_graph_writes_to():
     assert np.abs(eager.double().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
 
 
+def test_launchers_on_two_streams_do_not_disturb_each_other():
+    """The launchers are re-entrant: matvecs with k-split workspaces, layer transforms and the
+    batched product issued alternately on two streams (each stream its own outputs and its own
+    workspaces, as the wrappers hand them out) give the results of the same calls issued alone."""
+    import torch
+    from qtip_amd import ops
+    g = torch.Generator().manual_seed(11)
+    tl = torch.randn(512, 2, generator=g).half().cuda()
+    cases = []
+    for m, k, K in ((4096, 4096, 2), (2048, 11008, 3), (10240, 8192, 2), (1024, 28672, 4)):
+        pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+        x = torch.randn(k, generator=g).half().cuda()
+        X = torch.randn(8, k, generator=g).half().cuda()
+        cases.append((pk, x, X, m, k, K))
+
+    def work(c):
+        pk, x, X, m, k, K = c
+        return (ops.decompress_matvec(pk, x, tl, m, k, K, split_k=True),
+                ops.decompress_matvec_parts(pk, x, tl, m, k, K).sum(0),
+                ops.decompress_gemm(pk, X, tl, m, k, K))
+
+    alone = [work(c) for c in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [None] * len(cases)
+    for rep in range(6):
+        for i, c in enumerate(cases):
+            with torch.cuda.stream(streams[(i + rep) % 2]):
+                got[i] = work(c)
+        torch.cuda.synchronize()
+        for a, b in zip(alone, got):
+            for ta, tb in zip(a, b):
+                assert torch.equal(ta, tb)
+
+
 def test_instruction_rate_probe_runs_every_kind():
     """The measurement aid behind bench.py's issue-rate figures: every kind launches, fills its
     sink, and a full-rate instruction is measurably cheaper than the decode loop it is part of."""
