@@ -432,7 +432,9 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   const int upw_r = GROUP ? pick3(grp.upw_r, gi) : upw_r_;
   static_assert(!XHALF || (XLDS && !XFORM), "two-half staging is a form of the plain staged x");
   static_assert(!HALF || (XLDS && !XFORM && !XHALF && !GROUP), "half units exist for the plain form with x in LDS");
-  constexpr int FIRST = DEPTH > 2 ? 2 : 1;  // wave-loads requested before the table is built
+  // wave-loads requested before the table is built.  With half units both: a half wave-load is
+  // decoded in half the time, which no longer covers the latency of a load requested after the barrier.
+  constexpr int FIRST = (DEPTH > 2 || HALF) ? 2 : 1;
   extern __shared__ __align__(16) uint8_t smem[];
   uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
   float* part = reinterpret_cast<float*>(smem + kLut128Bytes);  // [2][kWaves][32]
@@ -1592,16 +1594,17 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
   // row blocks left over by the rounds of whole units, when they fill at most half a round of the
   // full grid: each is cut into its two row halves (see HALF at the kernel).  The half units follow
   // the whole ones in the same two-stage load pipeline, so the whole units must end on an even
-  // item.  Measured: 10240x8192 11.1 -> 9.9 us, 12288x4096 7.15 -> 6.75 us at 2 bits.  Not used
-  // where it measured slower: without a round of whole units before them (twice the workgroups
-  // and twice the stream for matrices that are latency-bound anyway: 4096x4096 4.8 -> 5.3 us) and
-  // at 3 and 4 bits (the doubled stream of the left-over blocks costs what the halved decode saves).
+  // item.  Measured at 2 bits: 10240x8192 11.1 -> 9.8 us, 12288x4096 7.15 -> 6.6 us, and matrices
+  // that do not fill one round - 4096x4096 4.8 -> 4.55 us, 4096x11008 7.9 -> 6.9 us (half the
+  // decode per workgroup on twice the workgroups).  At 3 and 4 bits the doubled stream of the
+  // left-over blocks costs what the halved decode saves (slower on the 4096-wide matrices, 2-4 %
+  // faster on 10240x8192 only), so those keep whole units.
   const int full_range = di.cus / S;
   const int left = full_range > 0 ? (m >> 5) % full_range : 0;
   const int whole = full_range > 0 ? (m >> 5) / full_range : 0;
   const bool even_items = (((wl_per + kWaves - 1) / kWaves) & 1) == 0;
-  if (bits == 2 && xbytes <= kMatvecXBytes && left > 0 && 2 * left <= full_range && whole >= 1 && even_items) {
-    const dim3 gh((unsigned)S, (unsigned)full_range);
+  if (bits == 2 && xbytes <= kMatvecXBytes && left > 0 && 2 * left <= full_range && (whole == 0 || even_items)) {
+    const dim3 gh((unsigned)S, (unsigned)(whole > 0 ? full_range : 2 * left));
     matvec_kernel<2, 2, true, 0, false, false, true><<<gh, kThreads, kMatvecLds + xbytes, st>>>(
         dst, p, xx, t, m, k, wl_per, whole, 2 * left);
     return (int)hipGetLastError();
