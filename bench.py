@@ -369,6 +369,7 @@ def main():
         result["gemm_4bit"] = gemm
 
     if "ceilings" in extras:
+        import bench_probe  # libqtip_probe.so: the measurement aids, a library of their own beside this script
         # what the memory system of this box delivers to simple kernels, next to the 8 TB/s nominal peak:
         # a 1 GiB device-to-device copy (read + write), a fill (write only), a BLAS dot product and the library's
         # own read probe (read only; the probe uses the matvec's persistent grid and non-temporal 16-byte loads)
@@ -379,7 +380,7 @@ def main():
         cases = {"copy_read_plus_write": (lambda: dst.copy_(src), 2 * nb),
                  "fill_write": (lambda: dst.fill_(1), nb),
                  "blas_dot_read": (lambda: torch.dot(fa, fb), nb),
-                 "stream_read": (lambda: ops.probe_stream_read(src), nb)}
+                 "stream_read": (lambda: bench_probe.stream_read(src), nb)}
         ceil = {}
         for name, (fn, moved) in cases.items():
             gr = capture(lambda: [fn() for _ in range(4)])
@@ -390,10 +391,10 @@ def main():
         # ns one wave-instruction (one wave-load) occupies a SIMD with 4 waves per SIMD, as in the matvec
         issue = {}
         iters = 2000
-        for name in ops.PROBE_KINDS:
-            gr = capture(lambda: ops.probe_issue(name, iters, tlut))
+        for name in bench_probe.KINDS:
+            gr = capture(lambda: bench_probe.issue(name, iters, tlut))
             t = timed(gr, 3, args.settle_ms / 6)
-            per = iters * 4 * (1 if name.startswith("decode_loop") else ops.PROBE_OPS_PER_ITER)
+            per = iters * 4 * (1 if name.startswith("decode_loop") else bench_probe.OPS_PER_ITER)
             issue[name] = round(t * 1e9 / per, 2 if per > iters * 4 else 1)
             del gr
         ceil["issue_ns_per_wave_instruction_and_simd"] = {k: v for k, v in issue.items() if not k.startswith("decode_loop")}

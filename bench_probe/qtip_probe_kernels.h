@@ -1,6 +1,7 @@
 // Measurement aids for the 2-bit matvec: the issue rate of the instructions its decode is made
-// of, and the decode loop by itself.  Included by qtip_hip.hip (which provides
-// matvec_accumulate and the table builders); nothing here runs on the product path.
+// of, and the decode loop by itself.  Included by qtip_probe.hip; the decode steps
+// (matvec_accumulate, the table builders) come from the product's own device header, so the
+// probe times the code the kernel runs.  Nothing here is part of libqtip_hip.so.
 //
 // issue_probe_kernel<KIND>: one workgroup of 16 waves per CU (4 waves per SIMD, as in the
 // matvec); every wave executes `iters` x 88 instructions of one kind on 8 independent registers,
@@ -12,6 +13,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include "../qtip_amd/csrc/qtip_device.h"
 
 namespace {
 

@@ -78,8 +78,6 @@ _SIGNATURES = {
                          [ctypes.c_long, ctypes.c_long, ctypes.c_void_p]),
     "qtip_sample_pick": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_uint] +
                          [ctypes.c_void_p] * 4 + [ctypes.c_long, ctypes.c_long, ctypes.c_void_p]),
-    "qtip_probe_stream_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
-    "qtip_probe_issue": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
     "qtip_repack": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "qtip_unpack_trellis": (ctypes.c_int, [ctypes.c_void_p] * 2 + [ctypes.c_long] + [ctypes.c_int] * 3 +
                             [ctypes.c_void_p]),

@@ -341,4 +341,58 @@ __device__ __forceinline__ uint32_t lds_word_abs(uint32_t lds_addr) {
   return *(lds_u32_t*)(uintptr_t)lds_addr;
 }
 
+// index into W[32] (lookup order of the packed hashes) of state (R, t, j)
+template <int K>
+__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
+  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
+  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
+}
+
+
+// 32 states of one wave-load.  All hashes, addresses and the 32 table reads are issued first, so
+// a read has the rest of the address arithmetic (a few hundred cycles) to come back from LDS;
+// the products run on the matrix core, which leaves the vector ALU to the decode (a v_dot2c per
+// state measured 5 % slower end to end).  The four table words of a
+// (tile row half mh, row half rh, kh) group are a v_mfma_f32_16x16x32_f16 B operand (N = the 16
+// lanes `a` of a DPP row, K group = g), the lane's own eight x values of that kh are the A operand
+// row `a`: D[i][j] = sum over (g, 8 halves) of x(lane i) * W(lane j), which is the wanted dot
+// product whenever lanes i and j read the same columns, i.e. i % 2 == j % 2.  Lane (g, a) keeps
+// D[4g + r][a] in element r, so element a % 2 of the accumulator is the lane's row sum over all
+// four blocks of the wave-load (the cross-block reduction happens inside the MFMA).
+//
+// RH = 0 / 1 decodes only the states of row half rh = RH (rows 8*RH .. 8*RH + 7 of either tile
+// row half): the registers P[i] with i % 2 == RH at every bit width, half the hashes, lookups and
+// MFMAs and - the extraction of the others being dead code - about half the vector work.  The
+// accumulators of the other row half stay untouched.
+template <int K, int RH = -1>
+__device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u32x2 xv[4],
+                                                       uint32_t slot4, float4_t acc[4]) {
+  uint32_t P[16], W[32];
+  packed_states<K>(ld, P);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if (RH >= 0 && (i & 1) != RH) continue;
+    const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
+    W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
+    W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int kh = 0; kh < 2; ++kh) {
+    const u32x4 xa = {xv[2 * kh][0], xv[2 * kh][1], xv[2 * kh + 1][0], xv[2 * kh + 1][1]};
+#pragma unroll
+    for (int mh = 0; mh < 2; ++mh)
+#pragma unroll
+      for (int rh = 0; rh < 2; ++rh) {
+        if (RH >= 0 && rh != RH) continue;
+        const int tt = 2 * kh + mh;
+        const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
+                          W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
+        acc[2 * mh + rh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            __builtin_bit_cast(half8_t, xa), __builtin_bit_cast(half8_t, wv), acc[2 * mh + rh], 0, 0, 0);
+      }
+  }
+}
+
 }  // namespace qtip

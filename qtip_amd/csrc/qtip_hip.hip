@@ -39,13 +39,6 @@ __device__ __forceinline__ float dpp_xor1(float v) {
 // ---------------------------------------------------------------------------
 constexpr size_t kDecodeLds = kLut128Bytes + kWaves * 2048;
 
-// index into W[32] (lookup order of the packed hashes) of state (R, t, j)
-template <int K>
-__device__ __forceinline__ constexpr int w_index(int R, int t, int j) {
-  if (K == 4) return 2 * ((R * 4 + t) * 2 + (j & 1)) + (1 - (j >> 1));
-  return 2 * ((R * 2 + (t >> 1)) * 4 + j) + (t & 1);
-}
-
 template <int K>
 __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restrict__ out,
                                                              const uint8_t* __restrict__ packed,
@@ -141,52 +134,6 @@ __global__ __launch_bounds__(kThreads, 1) void decode_kernel(uint16_t* __restric
 // ---------------------------------------------------------------------------
 constexpr size_t kMatvecLds = kLut128Bytes + 2 * kWaves * 32 * sizeof(float);
 constexpr size_t kMatvecXBytes = 28 * 1024;  // LDS left for the x values of a workgroup's k range
-
-// 32 states of one wave-load.  All hashes, addresses and the 32 table reads are issued first, so
-// a read has the rest of the address arithmetic (a few hundred cycles) to come back from LDS;
-// the products run on the matrix core, which leaves the vector ALU to the decode (a v_dot2c per
-// state measured 5 % slower end to end).  The four table words of a
-// (tile row half mh, row half rh, kh) group are a v_mfma_f32_16x16x32_f16 B operand (N = the 16
-// lanes `a` of a DPP row, K group = g), the lane's own eight x values of that kh are the A operand
-// row `a`: D[i][j] = sum over (g, 8 halves) of x(lane i) * W(lane j), which is the wanted dot
-// product whenever lanes i and j read the same columns, i.e. i % 2 == j % 2.  Lane (g, a) keeps
-// D[4g + r][a] in element r, so element a % 2 of the accumulator is the lane's row sum over all
-// four blocks of the wave-load (the cross-block reduction happens inside the MFMA).
-//
-// RH = 0 / 1 decodes only the states of row half rh = RH (rows 8*RH .. 8*RH + 7 of either tile
-// row half): the registers P[i] with i % 2 == RH at every bit width, half the hashes, lookups and
-// MFMAs and - the extraction of the others being dead code - about half the vector work.  The
-// accumulators of the other row half stay untouched.
-template <int K, int RH = -1>
-__device__ __forceinline__ void matvec_accumulate(const LaneData<K>& ld, const u32x2 xv[4],
-                                                       uint32_t slot4, float4_t acc[4]) {
-  uint32_t P[16], W[32];
-  packed_states<K>(ld, P);
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    if (RH >= 0 && (i & 1) != RH) continue;
-    const uint32_t q = pk_hash(P[i]) & 0xFFC0FFC0u;
-    W[2 * i] = lds_word_abs(lut128_addr_lo(q, slot4));
-    W[2 * i + 1] = lds_word_abs(lut128_addr_hi(q, slot4));
-  }
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int kh = 0; kh < 2; ++kh) {
-    const u32x4 xa = {xv[2 * kh][0], xv[2 * kh][1], xv[2 * kh + 1][0], xv[2 * kh + 1][1]};
-#pragma unroll
-    for (int mh = 0; mh < 2; ++mh)
-#pragma unroll
-      for (int rh = 0; rh < 2; ++rh) {
-        if (RH >= 0 && rh != RH) continue;
-        const int tt = 2 * kh + mh;
-        const u32x4 wv = {W[w_index<K>(0, tt, rh)], W[w_index<K>(1, tt, rh)],
-                          W[w_index<K>(0, tt, 2 + rh)], W[w_index<K>(1, tt, 2 + rh)]};
-        acc[2 * mh + rh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-            __builtin_bit_cast(half8_t, xa), __builtin_bit_cast(half8_t, wv), acc[2 * mh + rh], 0, 0, 0);
-      }
-  }
-}
 
 // Buffer-addressed streaming loads: the address is (SGPR descriptor, SGPR byte
 // offset, per-lane VGPR offset), so walking the stream costs no vector ALU work.
@@ -1324,9 +1271,6 @@ __global__ __launch_bounds__(256) void sum_parts_round_kernel(float* __restrict_
 constexpr size_t kScratchFloats = 64 * 1024;  // 256 KiB
 static __device__ __align__(256) float scratch[kScratchFloats];
 
-}  // namespace
-#include "qtip_probe.h"
-namespace {
 
 template <typename F>
 hipError_t allow_lds(F* fn, size_t bytes) {
@@ -1369,9 +1313,6 @@ hipError_t allow_lds_all() {
   QTIP_ALLOW((gemm_kernel<3, 2, 4, 8>), kGemmLds)
   QTIP_ALLOW((gemm4_kernel<1>), kGemm4Lds)
   QTIP_ALLOW((gemm4_kernel<2>), kGemm4Lds)
-  QTIP_ALLOW((issue_probe_kernel<kProbeDsRead>), kProbeLds)
-  QTIP_ALLOW((loop_probe_kernel<0>), kProbeLds)
-  QTIP_ALLOW((loop_probe_kernel<1>), kProbeLds)
 #undef QTIP_ALLOW
   return hipSuccess;
 }
@@ -1977,37 +1918,5 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   }
   return QTIP_OK;
 }
-
-int qtip_probe_issue(int kind, int iters, const void* tlut, void* sink_u32, void* stream) {
-  if (!tlut || !sink_u32) return QTIP_E_NULL;
-  if (iters < 1 || iters > (1 << 20)) return QTIP_E_SHAPE;
-  if (const int rc = ready_code(stream)) return rc;
-  const DeviceInfo di = device_info();
-  hipStream_t st = (hipStream_t)stream;
-  const uint32_t* tl = (const uint32_t*)tlut;
-  uint32_t* sink = (uint32_t*)sink_u32;
-  switch (kind) {
-#define QTIP_PROBE(KIND, LDS) \
-  case KIND: issue_probe_kernel<KIND><<<di.cus, 1024, LDS, st>>>(iters, tl, sink); break;
-    QTIP_PROBE(kProbeAnd, 0)
-    QTIP_PROBE(kProbeAddU32, 0)
-    QTIP_PROBE(kProbeLshrImm, 0)
-    QTIP_PROBE(kProbeLshlImm, 0)
-    QTIP_PROBE(kProbePkMad, 0)
-    QTIP_PROBE(kProbeMadU32U16, 0)
-    QTIP_PROBE(kProbePerm, 0)
-    QTIP_PROBE(kProbePkLshr, 0)
-    QTIP_PROBE(kProbeMovDpp, 0)
-    QTIP_PROBE(kProbeDot2c, 0)
-    QTIP_PROBE(kProbeDsRead, kProbeLds)
-    QTIP_PROBE(kProbeMfma, 0)
-#undef QTIP_PROBE
-    case kProbeLoop: loop_probe_kernel<0><<<di.cus, 1024, kProbeLds, st>>>(iters, tl, sink); break;
-    case kProbeLoopValu: loop_probe_kernel<1><<<di.cus, 1024, kProbeLds, st>>>(iters, tl, sink); break;
-    default: return QTIP_E_SHAPE;
-  }
-  return (int)hipGetLastError();
-}
-
 
 }  // extern "C"

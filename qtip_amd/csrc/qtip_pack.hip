@@ -214,44 +214,3 @@ int qtip_decode_natural(void* out, const void* packed, const void* lut, int lut_
 
 
 }  // extern "C"
-
-namespace {
-// Read `n16` 16-byte words once with the loads of the matvec's stream (non-temporal dwordx4,
-// one per lane, persistent workgroups) and fold them into one word per wave.
-typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(1024) void stream_read_probe_kernel(uint32_t* __restrict__ sink,
-                                                                 const probe_u32x4* __restrict__ src, size_t n16) {
-  const size_t nthreads = (size_t)gridDim.x * blockDim.x;
-  uint32_t acc = 0;
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 3 * nthreads < n16; i += 4 * nthreads) {
-    const probe_u32x4 a = __builtin_nontemporal_load(src + i);
-    const probe_u32x4 b = __builtin_nontemporal_load(src + i + nthreads);
-    const probe_u32x4 c = __builtin_nontemporal_load(src + i + 2 * nthreads);
-    const probe_u32x4 d = __builtin_nontemporal_load(src + i + 3 * nthreads);
-    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
-  }
-  for (; i < n16; i += nthreads) {
-    const probe_u32x4 a = __builtin_nontemporal_load(src + i);
-    acc ^= a.x ^ a.y ^ a.z ^ a.w;
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o);
-  if ((threadIdx.x & 63) == 0) sink[(size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)] = acc;
-}
-}  // namespace
-
-extern "C" {
-
-int qtip_probe_stream_read(void* sink_u32, const void* src, size_t bytes, void* stream) {
-  if (!sink_u32 || !src) return QTIP_E_NULL;
-  if (bytes < 16 || !aligned(src, 16)) return QTIP_E_ALIGN;
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
-    return (int)hipErrorInvalidDevice;
-  stream_read_probe_kernel<<<cus, 1024, 0, (hipStream_t)stream>>>((uint32_t*)sink_u32, (const probe_u32x4*)src, bytes / 16);
-  return (int)hipGetLastError();
-}
-
-}  // extern "C"

@@ -577,39 +577,6 @@ def greedy_pick(logits, tok, pos, history=None, history_base=0):
                                      stream_ptr(logits.device)), "qtip_greedy_pick")
 
 
-def probe_stream_read(src):
-    """Read the tensor once with the matvec's kind of loads (measurement aid: the launch's duration
-    is the stream-read ceiling bench.py reports).  Returns the per-wave folded words."""
-    require_cuda(src, "src")
-    cus = torch.cuda.get_device_properties(src.device).multi_processor_count
-    sink = torch.empty(16 * cus, dtype=torch.int32, device=src.device)
-    with torch.cuda.device(src.device):
-        check(lib().qtip_probe_stream_read(_ptr(sink), _ptr(src), src.numel() * src.element_size(),
-                                           stream_ptr(src.device)), "qtip_probe_stream_read")
-    return sink
-
-
-PROBE_OPS_PER_ITER = 88
-PROBE_KINDS = {"v_and_b32": 0, "v_add_u32": 1, "v_lshrrev_b32": 2, "v_lshlrev_b32": 3, "v_pk_mad_u16": 4,
-               "v_mad_u32_u16": 5, "v_perm_b32": 6, "v_pk_lshrrev_b16": 7, "v_mov_b32_dpp": 8, "v_dot2c_f32_f16": 9,
-               "ds_read_b32": 10, "v_mfma_f32_16x16x32_f16": 11, "decode_loop": 100, "decode_loop_valu": 101}
-
-
-def probe_issue(kind, iters, tlut, sink=None):
-    """One launch of the instruction-rate probe (measurement aid): `kind` a key of PROBE_KINDS.
-    The caller times it; see include/qtip_hip.h for what a launch executes."""
-    require_cuda(tlut, "tlut", torch.float16)
-    if tlut.numel() != 1024:
-        raise ValueError("tlut holds 512 x 2 fp16 values")
-    cus = torch.cuda.get_device_properties(tlut.device).multi_processor_count
-    if sink is None:
-        sink = torch.empty(1024 * cus, dtype=torch.int32, device=tlut.device)
-    with torch.cuda.device(tlut.device):
-        check(lib().qtip_probe_issue(PROBE_KINDS[kind], int(iters), _ptr(tlut), _ptr(sink), stream_ptr(tlut.device)),
-              "qtip_probe_issue")
-    return sink
-
-
 SAMPLE_PICK_MAX_TOP_K = 64
 
 

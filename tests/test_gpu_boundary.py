@@ -125,32 +125,3 @@ def test_launchers_on_two_streams_do_not_disturb_each_other():
         for a, b in zip(alone, got):
             for ta, tb in zip(a, b):
                 assert torch.equal(ta, tb)
-
-
-def test_instruction_rate_probe_runs_every_kind():
-    """The measurement aid behind bench.py's issue-rate figures: every kind launches, fills its
-    sink, and a full-rate instruction is measurably cheaper than the decode loop it is part of."""
-    import torch
-    from qtip_amd import ops
-    tlut = torch.randn(512, 2, generator=torch.Generator().manual_seed(0)).half().cuda()
-    cus = torch.cuda.get_device_properties(0).multi_processor_count
-    times = {}
-    for name in ops.PROBE_KINDS:
-        sink = torch.full((1024 * cus,), -1, dtype=torch.int32, device="cuda")
-        ops.probe_issue(name, 20, tlut, sink)  # warm
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        ops.probe_issue(name, 400, tlut, sink)
-        e1.record()
-        torch.cuda.synchronize()
-        times[name] = e0.elapsed_time(e1)
-        assert times[name] > 0
-    per_op = times["v_and_b32"] * 1e6 / (400 * ops.PROBE_OPS_PER_ITER * 4)
-    per_item = times["decode_loop"] * 1e6 / (400 * 4)
-    assert 0.2 < per_op < 20 and 50 < per_item < 2000, (per_op, per_item)
-    assert times["decode_loop_valu"] < times["decode_loop"]
-    with pytest.raises(KeyError):
-        ops.probe_issue("v_nop", 10, tlut)
-    from qtip_amd import _lib
-    rc = _lib.lib().qtip_probe_issue(55, 10, tlut.data_ptr(), sink.data_ptr(), None)
-    assert rc == -1  # an unknown kind is a shape error, nothing is launched

@@ -764,15 +764,6 @@ def test_silu_pair_rejects_what_it_does_not_cover():
                           had_bits=torch.zeros(1, dtype=torch.int32, device="cuda"))
 
 
-def test_stream_read_probe_reads_every_word_once():
-    from qtip_amd import ops
-    for n16 in (4, 4099, 1 << 18):
-        src = torch.randint(-2**31, 2**31 - 1, (n16 * 4,), dtype=torch.int32,
-                            generator=torch.Generator().manual_seed(n16))
-        sink = ops.probe_stream_read(src.cuda()).cpu().numpy()
-        assert int(np.bitwise_xor.reduce(sink)) == int(np.bitwise_xor.reduce(src.numpy()))
-
-
 def test_token_head_kernels():
     """Final RMSNorm against the module's formula (model/llama.py:129-135) and the greedy pick
     against torch.argmax: first index among equal maxima, history slot, advanced position."""

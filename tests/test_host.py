@@ -29,6 +29,22 @@ def test_library_exports_every_declared_symbol():
     assert b"shape" in _lib.lib().qtip_error_string(-1)
 
 
+def test_measurement_aids_live_in_a_library_of_their_own():
+    """libqtip_hip.so exports no probe; bench_probe/libqtip_probe.so exports what its header declares."""
+    from qtip_amd import _lib
+    import bench_probe
+    main = ctypes.CDLL(_lib.LIB_PATH)
+    assert os.path.exists(bench_probe.LIB_PATH), "build with python -m bench_probe"
+    probe = ctypes.CDLL(bench_probe.LIB_PATH)
+    text = open(os.path.join(ROOT, "bench_probe", "qtip_probe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(qtip_probe_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["qtip_probe_issue", "qtip_probe_stream_read"]
+    for name in names:
+        assert hasattr(probe, name), name
+        assert not hasattr(main, name), name
+
+
 def test_argument_rejection_without_gpu():
     # rejected arguments return a negative code before anything touches the device
     from qtip_amd import _lib
