@@ -99,10 +99,11 @@ int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16,
  * library's own device image (one copy per GPU, held until the process ends), so the call
  * allocates nothing: no hipMalloc / hipFree, no workspace argument.
  *   nparts = 0: the library's choice of k split (the one qtip_decompress_matvec makes with a
- *               workspace); 1..16: that many k ranges.
+ *               workspace, halved until its partial sums fit the array: never an error);
+ *               1..16: that many k ranges.
  * Results are bit-identical to qtip_decompress_matvec with the same split.
- * Limit: nparts * m <= 65536 floats, else QTIP_E_SCRATCH (nothing launched; nparts = 1 never
- * needs the scratch).  The partial sums are all written before they are read, so nothing has to
+ * Limit for a split the caller asks for: nparts * m <= 65536 floats, else QTIP_E_SCRATCH
+ * (nothing launched; nparts = 1 never needs the scratch).  The partial sums are all written before they are read, so nothing has to
  * be cleared between calls; but every call on a GPU uses that GPU's one array: calls that
  * overlap in time on one GPU (different streams, or graphs replayed concurrently) race. */
 int qtip_decompress_matvec_noalloc(float* out, const void* packed, const void* x_f16,

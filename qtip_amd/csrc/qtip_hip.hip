@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -626,13 +627,15 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       if (t + d < t1 && c_j == npw) {
         // ---- end of a unit: ragged tail, reductions, store
         // k/32 not a multiple of 4: one wave takes the partial wave-load.  Every lane takes part
-        // in an MFMA, so the lanes of the missing blocks read x = 0 (the descriptor of x ends
-        // at k) and whatever follows in the stream (0 past its end).
+        // in an MFMA, so the lanes of the missing tile blocks (g >= nkb % 4) load x and the stream
+        // with a lane offset that is out of range by itself: both come back as zeros without a
+        // memory access, whatever the range check makes of the scalar offset.
         if (tail_wave) {
+          const bool in_row = g < nkb - 4 * nfull;
           u32x2 xt[4];
-          load_x_buf(rs_x, xoff, (uint32_t)nfull * 256u, xt);
-          const LaneData<K> tail =
-              load_lane_buf<K>(rs_w, loff, (uint32_t)c_rb * rb_bytes + (uint32_t)nfull * WL_BYTES);
+          load_x_buf(rs_x, in_row ? xoff : 0x7FFFFF00u, (uint32_t)nfull * 256u, xt);
+          const LaneData<K> tail = load_lane_buf<K>(rs_w, in_row ? loff : 0x7FFFFF00u,
+                                                    (uint32_t)c_rb * rb_bytes + (uint32_t)nfull * WL_BYTES);
           accumulate(tail, xt);
         }
         float* pp = part + parity * (kWaves * 32);
@@ -765,7 +768,10 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_kernel(
     const int rb = l_grp * kGemmRB + rbi;
     const int wl = wl0 + KS * l_t + ks;
     const bool valid = l_q < T && rb < nrb && wl < wl1;
-    buf[d] = load_lane_buf<K>(rs_w, valid ? loff : 0x7FFFFF00u,  // padding: out of range, no memory access
+    // padding items, and the lanes past the row's end in a partial last wave-load (k / 32 not a
+    // multiple of 4): a lane offset that is out of range by itself, zeros without a memory access
+    const bool lane_ok = valid && 4 * wl + g < nkb;
+    buf[d] = load_lane_buf<K>(rs_w, lane_ok ? loff : 0x7FFFFF00u,
                               valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u);
     ++l_q;
     if (++l_t == nst) {
@@ -1052,7 +1058,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm4_kernel(
     const int rb = l_grp * kGemmRB + rbi;
     const int wl = wl0 + KS * l_t + ks;
     const bool valid = l_q < T && rb < nrb && wl < wl1;
-    const uint32_t vo = valid ? loff : 0x7FFFFF00u;  // padding: out of range, no memory access
+    // padding items, and the lanes past the row's end in a partial last wave-load: a lane offset
+    // that is out of range by itself, zeros without a memory access
+    const uint32_t vo = (valid && 4 * wl + g < nkb) ? loff : 0x7FFFFF00u;
     const uint32_t so = valid ? (uint32_t)rb * rb_bytes + (uint32_t)wl * WL_BYTES : 0u;
 #pragma unroll
     for (int cp = 0; cp < 4; ++cp) {
@@ -1325,40 +1333,37 @@ hipError_t allow_lds_all() {
 struct DeviceState {
   int cus = 0;
   float* scratch_ptr = nullptr;
-  hipError_t status = hipErrorNotInitialized;
-  bool done = false;
-  bool refused = false;  // first use of the device inside a stream capture: set-up not run
+  std::atomic<bool> done{false};  // set last, read first: the fields above are complete when it is true
 };
 constexpr int kMaxDevices = 64;
 DeviceState g_devices[kMaxDevices];
 std::mutex g_devices_mutex;
 
-// A launcher that meets a device for the first time while its stream is being captured does
-// not run the set-up (hipFuncSetAttribute and friends are no calls to make inside a capture):
-// it reports QTIP_E_NOT_INIT (`refused` in the state it gets back).
+// What a launcher learns about its device in one look: rc = 0, QTIP_E_NOT_INIT (first use of the
+// device inside a stream capture: the set-up is not run there and nothing is launched) or the
+// hipError_t of a failed set-up (tried again by the next call).
+struct Ready {
+  int rc;
+  int cus;
+  float* scratch;
+};
 
-// State of the current device, set up on first use; status != hipSuccess if that failed.
-// `launching`: the caller is about to enqueue work on `st`.
-DeviceState& device_state(bool launching = false, hipStream_t st = nullptr) {
-  static thread_local DeviceState none;  // no usable device / refused: status is an error
+// State of the current device, set up on first use.  `launching`: the caller is about to
+// enqueue work on `st`.  One hipGetDevice per call; the mutex only on the first use of a device.
+Ready ready(bool launching, hipStream_t st) {
   int dev = -1;
   const hipError_t ge = hipGetDevice(&dev);
-  if (ge != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-    none.status = ge != hipSuccess ? ge : hipErrorInvalidDevice;
-    none.refused = false;
-    return none;
-  }
-  std::lock_guard<std::mutex> lock(g_devices_mutex);
+  if (ge != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return Ready{(int)(ge != hipSuccess ? ge : hipErrorInvalidDevice), 0, nullptr};
   DeviceState& d = g_devices[dev];
-  if (d.done) return d;
+  if (d.done.load(std::memory_order_acquire)) return Ready{0, d.cus, d.scratch_ptr};
+  std::lock_guard<std::mutex> lock(g_devices_mutex);
+  if (d.done.load(std::memory_order_relaxed)) return Ready{0, d.cus, d.scratch_ptr};
   if (launching) {
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     const hipError_t ce = hipStreamIsCapturing(st, &cs);
-    if (ce == hipErrorStreamCaptureImplicit || (ce == hipSuccess && cs != hipStreamCaptureStatusNone)) {
-      none.status = hipErrorNotInitialized;
-      none.refused = true;
-      return none;
-    }
+    if (ce == hipErrorStreamCaptureImplicit || (ce == hipSuccess && cs != hipStreamCaptureStatusNone))
+      return Ready{QTIP_E_NOT_INIT, 0, nullptr};
     if (ce != hipSuccess) (void)hipGetLastError();  // the query's own error is not the caller's
   }
   int cus = 0;
@@ -1367,28 +1372,23 @@ DeviceState& device_state(bool launching = false, hipStream_t st = nullptr) {
   float* sp = nullptr;
   if (e == hipSuccess) e = hipGetSymbolAddress(reinterpret_cast<void**>(&sp), HIP_SYMBOL(scratch));
   if (e == hipSuccess && !sp) e = hipErrorInvalidSymbol;
-  d.status = e;
-  if (e == hipSuccess) {
-    d.cus = cus > 0 ? cus : 256;
-    d.scratch_ptr = sp;
-    d.done = true;  // a failed set-up is tried again by the next call
-  }
-  return d;
+  if (e != hipSuccess) return Ready{(int)e, 0, nullptr};
+  d.cus = cus > 0 ? cus : 256;
+  d.scratch_ptr = sp;
+  d.done.store(true, std::memory_order_release);
+  return Ready{0, d.cus, d.scratch_ptr};
 }
+Ready ready(void* stream) { return ready(true, (hipStream_t)stream); }
 
-// the launchers below read the CU count through this view
-struct DeviceInfo {
-  int cus;
-  bool ok;
-};
-DeviceInfo device_info() {
-  const DeviceState& d = device_state();
-  return DeviceInfo{d.cus, d.status == hipSuccess};
-}
-// return code of a launcher for the state of its device: 0, QTIP_E_NOT_INIT or a hipError_t
-int ready_code(void* stream) {
-  const DeviceState& d = device_state(true, (hipStream_t)stream);
-  return d.refused ? QTIP_E_NOT_INIT : (int)d.status;
+// CU count of the current device for the size queries: no set-up (they may be a process's first
+// call on the device and may come while a stream is being captured), 0 when there is no device.
+int query_cus() {
+  int dev = -1, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  const DeviceState& d = g_devices[dev];
+  if (d.done.load(std::memory_order_acquire)) return d.cus;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  return cus > 0 ? cus : 256;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1439,7 +1439,7 @@ extern "C" {
 
 int qtip_abi_version(void) { return 20; }
 
-int qtip_init(void) { return (int)device_state().status; }
+int qtip_init(void) { return ready(false, nullptr).rc; }
 
 const char* qtip_error_string(int code) {
   switch (code) {
@@ -1465,8 +1465,8 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
   if (rc) return rc;
   if (!aligned16(out_f16) || !aligned16(packed) || (reinterpret_cast<uintptr_t>(tlut) & 3u))
     return QTIP_E_ALIGN;
-  if ((rc = ready_code(stream))) return rc;
-  const DeviceInfo di = device_info();
+  const Ready di = ready(stream);
+  if (di.rc) return di.rc;
   const long total = (long)(m >> 5) * (((k >> 5) + 3) >> 2);
   long want = (total + kWaves - 1) / kWaves;
   const int grid = (int)(want < di.cus ? want : di.cus);
@@ -1484,23 +1484,21 @@ int qtip_decode(void* out_f16, const void* packed, const void* tlut, int m, int 
 
 int qtip_matvec_split(int m, int k, int bits) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
-  const DeviceInfo di = device_info();
-  if (!di.ok) return 0;
-  return choose_split(m, k, bits, di.cus, false);
+  const int cus = query_cus();
+  return cus ? choose_split(m, k, bits, cus, false) : 0;
 }
 
 size_t qtip_matvec_workspace_bytes(int m, int k, int bits) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4) return 0;
-  const DeviceInfo di = device_info();
-  if (!di.ok) return 0;
-  const int S = choose_split(m, k, bits, di.cus, true);
+  const int cus = query_cus();
+  if (!cus) return 0;
+  const int S = choose_split(m, k, bits, cus, true);
   return S > 1 ? (size_t)S * m * sizeof(float) : 0;
 }
 
-static int launch_matvec(float* dst, const void* packed, const void* x_f16, const void* tlut, int m,
-                         int k, int bits, int S, hipStream_t st, const void* su_f16 = nullptr,
+static int launch_matvec(const Ready& di, float* dst, const void* packed, const void* x_f16, const void* tlut,
+                         int m, int k, int bits, int S, hipStream_t st, const void* su_f16 = nullptr,
                          float xscale = 1.f, const ChainArgs* chain = nullptr) {
-  const DeviceInfo di = device_info();
   const long units = (long)(m >> 5) * S;
   long grid = units < di.cus ? units : di.cus;
   grid -= grid % S;  // a workgroup keeps one k range (units is a multiple of S, so grid >= S)
@@ -1576,34 +1574,38 @@ static int launch_matvec(float* dst, const void* packed, const void* x_f16, cons
 }
 
 static int check_matvec(const void* out, const void* packed, const void* x_f16, const void* tlut,
-                        int m, int k, int bits, void* stream) {
+                        int m, int k, int bits) {
   int rc = check_common(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (!aligned16(packed) || (reinterpret_cast<uintptr_t>(x_f16) & 7u) ||
       (reinterpret_cast<uintptr_t>(tlut) & 3u) || (reinterpret_cast<uintptr_t>(out) & 3u))
     return QTIP_E_ALIGN;
-  return ready_code(stream);
+  return QTIP_OK;
 }
 
 int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x_f16,
                                  const void* tlut, int m, int k, int bits, int nparts,
                                  void* stream) {
-  int rc = check_matvec(parts, packed, x_f16, tlut, m, k, bits, stream);
+  int rc = check_matvec(parts, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (nparts < 1 || nparts > kMaxSplit || nparts > ((((k >> 5) + 3) >> 2))) return QTIP_E_SHAPE;
-  return launch_matvec(parts, packed, x_f16, tlut, m, k, bits, nparts, (hipStream_t)stream);
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
+  return launch_matvec(rd, parts, packed, x_f16, tlut, m, k, bits, nparts, (hipStream_t)stream);
 }
 
 int qtip_decompress_matvec_parts_rht(float* parts, const void* packed, const void* x_raw_f16,
                                      const void* su_f16, float scale, const void* tlut, int m, int k,
                                      int bits, int nparts, void* stream) {
-  int rc = check_matvec(parts, packed, x_raw_f16, tlut, m, k, bits, stream);
+  int rc = check_matvec(parts, packed, x_raw_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (!su_f16) return QTIP_E_NULL;
   if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
   if (nparts < 1 || nparts > kMaxSplit || nparts > (k >> 7)) return QTIP_E_SHAPE;
   if (!aligned16(x_raw_f16) || !aligned16(su_f16)) return QTIP_E_ALIGN;
-  return launch_matvec(parts, packed, x_raw_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale);
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
+  return launch_matvec(rd, parts, packed, x_raw_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale);
 }
 
 int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const void* tlut, int m, int k,
@@ -1612,7 +1614,7 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
                                        const void* residual_f16, const void* norm_w_f16, float eps,
                                        const void* su_f16, float scale_in, void* x_out_f16,
                                        void* stream) {
-  int rc = check_matvec(parts, packed, su_f16, tlut, m, k, bits, stream);
+  int rc = check_matvec(parts, packed, su_f16, tlut, m, k, bits);
   if (rc) return rc;
   if (!prev_parts || !post || !residual_f16 || !norm_w_f16 || !x_out_f16) return QTIP_E_NULL;
   if (k != 2048 && k != 4096 && k != 8192) return QTIP_E_SHAPE;
@@ -1631,7 +1633,9 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
   c.scale_out = scale_out;
   c.eps = eps;
   c.in_parts = prev_nparts;
-  return launch_matvec(parts, packed, su_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale_in, &c);
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
+  return launch_matvec(rd, parts, packed, su_f16, tlut, m, k, bits, nparts, (hipStream_t)stream, su_f16, scale_in, &c);
 }
 
 }  // extern "C"
@@ -1640,9 +1644,9 @@ int qtip_decompress_matvec_parts_chain(float* parts, const void* packed, const v
 // their row blocks (at least one each, never more than a matrix has row blocks); fills every
 // field of GroupArgs except the pointers' meaning-specific ones (su / x).  Returns the number of
 // workgroups per k range, 0 if the device is too small for the group.
-static int share_out_group(GroupArgs& ga, float* parts, int ngroups, const void* const* packed,
+static int share_out_group(int cus, GroupArgs& ga, float* parts, int ngroups, const void* const* packed,
                            const void* const* tlut, const int* m, int S, long m_total) {
-  const int P = device_info().cus / S;
+  const int P = cus / S;
   if (P < ngroups) return 0;
   int nrb[3] = {0, 0, 0}, wg[3] = {0, 0, 0};
   long nrb_total = 0;
@@ -1717,7 +1721,7 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
   if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
   long m_total = 0;
   for (int g = 0; g < ngroups; ++g) {
-    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits, stream);
+    int rc = check_matvec(parts, packed[g], su_f16[g], tlut[g], m[g], k, bits);
     if (rc) return rc;
     if (!aligned16(su_f16[g])) return QTIP_E_ALIGN;
     m_total += m[g];
@@ -1741,8 +1745,10 @@ int qtip_decompress_matvec_group_chain(float* parts, int ngroups, const void* co
   c.in_parts = prev_nparts;
 
   const int S = nparts;
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
   GroupArgs ga;
-  const int used = share_out_group(ga, parts, ngroups, packed, tlut, m, S, m_total);
+  const int used = share_out_group(rd.cus, ga, parts, ngroups, packed, tlut, m, S, m_total);
   if (used == 0) return QTIP_E_SHAPE;
   for (int g = 0; g < 3; ++g) ga.su[g] = (const uint16_t*)su_f16[g < ngroups ? g : ngroups - 1];
   const int nwl = ((k >> 5) + 3) >> 2;
@@ -1765,7 +1771,7 @@ int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* p
   if (ngroups < 1 || ngroups > 3) return QTIP_E_SHAPE;
   long m_total = 0;
   for (int g = 0; g < ngroups; ++g) {
-    int rc = check_matvec(parts, packed[g], x_f16[g], tlut[g], m[g], k, bits, stream);
+    int rc = check_matvec(parts, packed[g], x_f16[g], tlut[g], m[g], k, bits);
     if (rc) return rc;
     if (!aligned16(x_f16[g])) return QTIP_E_ALIGN;
     m_total += m[g];
@@ -1776,8 +1782,10 @@ int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* p
   const int wl_per = (nwl + S - 1) / S;
   const size_t xbytes = (size_t)wl_per * 256;
   if (xbytes > kMatvecXBytes) return QTIP_E_SHAPE;  // the grouped plain form keeps x in LDS
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
   GroupArgs ga;
-  const int used = share_out_group(ga, parts, ngroups, packed, tlut, m, S, m_total);
+  const int used = share_out_group(rd.cus, ga, parts, ngroups, packed, tlut, m, S, m_total);
   if (used == 0) return QTIP_E_SHAPE;
   for (int g = 0; g < 3; ++g) ga.x[g] = (const uint16_t*)x_f16[g < ngroups ? g : ngroups - 1];
   const dim3 g2((unsigned)S, (unsigned)used);
@@ -1794,17 +1802,19 @@ int qtip_decompress_matvec_group(float* parts, int ngroups, const void* const* p
 int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, const void* tlut,
                            int m, int k, int bits, void* workspace, size_t workspace_bytes,
                            void* stream) {
-  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits, stream);
+  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
   int S = 1;
   if (workspace) {
-    S = choose_split(m, k, bits, device_info().cus, true);
+    S = choose_split(m, k, bits, rd.cus, true);
     if (S > 1 && workspace_bytes < (size_t)S * m * sizeof(float)) return QTIP_E_WORKSPACE;
     if (!aligned16(workspace)) return QTIP_E_ALIGN;
   }
   hipStream_t st = (hipStream_t)stream;
-  if (S == 1) return launch_matvec(out, packed, x_f16, tlut, m, k, bits, 1, st);
-  rc = launch_matvec((float*)workspace, packed, x_f16, tlut, m, k, bits, S, st);
+  if (S == 1) return launch_matvec(rd, out, packed, x_f16, tlut, m, k, bits, 1, st);
+  rc = launch_matvec(rd, (float*)workspace, packed, x_f16, tlut, m, k, bits, S, st);
   if (rc) return rc;
   sum_parts_kernel<<<(m + 255) / 256, 256, 0, st>>>(out, (const float*)workspace, m, S);
   return (int)hipGetLastError();
@@ -1812,18 +1822,24 @@ int qtip_decompress_matvec(float* out, const void* packed, const void* x_f16, co
 
 int qtip_decompress_matvec_noalloc(float* out, const void* packed, const void* x_f16, const void* tlut,
                                    int m, int k, int bits, int nparts, void* stream) {
-  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits, stream);
+  int rc = check_matvec(out, packed, x_f16, tlut, m, k, bits);
   if (rc) return rc;
-  const DeviceState& ds = device_state();  // set up by check_matvec (or qtip_init) already
+  const Ready rd = ready(stream);
+  if (rd.rc) return rd.rc;
   const int nwl = ((k >> 5) + 3) >> 2;
   if (nparts < 0 || nparts > kMaxSplit || nparts > nwl) return QTIP_E_SHAPE;
-  const int S = nparts ? nparts : choose_split(m, k, bits, ds.cus, true);
+  int S = nparts;
+  if (S == 0) {
+    // the library's own choice, halved until its partial sums fit the scratch (S = 1 needs none)
+    S = choose_split(m, k, bits, rd.cus, true);
+    while (S > 1 && (size_t)S * m > kScratchFloats) S >>= 1;
+  }
   hipStream_t st = (hipStream_t)stream;
-  if (S == 1) return launch_matvec(out, packed, x_f16, tlut, m, k, bits, 1, st);
-  if ((size_t)S * m > kScratchFloats) return QTIP_E_SCRATCH;
+  if (S == 1) return launch_matvec(rd, out, packed, x_f16, tlut, m, k, bits, 1, st);
+  if ((size_t)S * m > kScratchFloats) return QTIP_E_SCRATCH;  // only a split the caller asked for
   // every one of the S * m partial sums is written before it is read: nothing to clear
-  float* parts = ds.scratch_ptr;
-  rc = launch_matvec(parts, packed, x_f16, tlut, m, k, bits, S, st);
+  float* parts = rd.scratch;
+  rc = launch_matvec(rd, parts, packed, x_f16, tlut, m, k, bits, S, st);
   if (rc) return rc;
   sum_parts_kernel<<<(m + 255) / 256, 256, 0, st>>>(out, parts, m, S);
   return (int)hipGetLastError();
@@ -1841,9 +1857,9 @@ static int gemm_split(int m, int k, int cus) {
 
 size_t qtip_gemm_workspace_bytes(int m, int k, int bits, int batch) {
   if (m <= 0 || k <= 0 || (m & 31) || (k & 31) || bits < 2 || bits > 4 || batch < 1) return 0;
-  const DeviceInfo di = device_info();
-  if (!di.ok) return 0;
-  const int S = gemm_split(m, k, di.cus);
+  const int cus = query_cus();
+  if (!cus) return 0;
+  const int S = gemm_split(m, k, cus);
   return S > 1 ? (size_t)S * (batch < 32 ? batch : 32) * m * sizeof(float) : 0;
 }
 
@@ -1856,8 +1872,8 @@ int qtip_decompress_gemm(float* out, const void* packed, const void* x_f16, cons
   if (!aligned16(packed) || !aligned16(x_f16) || (reinterpret_cast<uintptr_t>(tlut) & 3u) ||
       (reinterpret_cast<uintptr_t>(out) & 3u))
     return QTIP_E_ALIGN;
-  if ((rc = ready_code(stream))) return rc;
-  const DeviceInfo di = device_info();
+  const Ready di = ready(stream);
+  if (di.rc) return di.rc;
   int S = 1;
   if (workspace) {
     S = gemm_split(m, k, di.cus);

@@ -9,6 +9,7 @@ kernel launch.  The order-K tables are the reference's
 hadamard_tables.npz.
 """
 import os
+import weakref
 
 import numpy as np
 import torch
@@ -73,11 +74,15 @@ def had_bits(hadK, K, transpose, device):
             neg = _table_signs(K).astype(bool)
             _bit_cache[key] = torch.from_numpy(_pack_bits(neg.T if transpose else neg)).to(dev)
         return _bit_cache[key]
-    # a caller's own table: the cache entry keeps the tensor alive, so its address cannot be handed to
-    # another tensor while the entry exists, and remembers the version it was packed from
-    key = (hadK.data_ptr(), tuple(hadK.shape), tuple(hadK.stride()), bool(transpose), dev)
+    # a caller's own table: keyed by the memory it occupies, so a fresh view of the same table (what
+    # a module hands in on every call) hits.  The entry holds a weak reference to the storage: while
+    # that storage lives its address cannot belong to another tensor, and when it is freed the entry
+    # goes with it (nothing of the caller's is kept alive).  An in-place change bumps `_version`.
+    st = hadK.untyped_storage()
+    key = (st.data_ptr(), hadK.storage_offset(), tuple(hadK.shape), tuple(hadK.stride()), hadK.dtype,
+           bool(transpose), dev)
     hit = _bit_cache.get(key)
-    if hit is None or hit[0] is not hadK or hit[1] != hadK._version:
+    if hit is None or hit[0]() is not st or hit[1] != hadK._version:
         h = hadK.detach().to("cpu", torch.float32).numpy()
         if h.shape != (K, K) or not np.all(np.abs(h) == 1.0):
             raise ValueError("hadK must be a K x K matrix of +-1")
@@ -87,7 +92,9 @@ def had_bits(hadK, K, transpose, device):
             bits = had_bits(None, K, transpose, dev)
         else:
             bits = torch.from_numpy(_pack_bits(neg.T if transpose else neg)).to(dev)
-        hit = (hadK, hadK._version, bits)
+        if hit is None or hit[0]() is not st:
+            weakref.finalize(st, _bit_cache.pop, key, None)
+        hit = (weakref.ref(st), hadK._version, bits)
         _bit_cache[key] = hit
     return hit[2]
 

@@ -84,6 +84,46 @@ def test_matvec_with_left_over_row_blocks_cut_by_row_half(m, k, nparts):
         assert_close(parts[0].cpu().numpy(), c_oracle.matvec(L["packed"], half, L["tlut"], m, k, K))
 
 
+@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("m,k", [(512, 4000), (256, 96), (10240, 4000)])
+def test_ragged_k_reads_nothing_behind_its_operands(m, k, K):
+    """k / 32 not a multiple of 4: the last wave-load of a row block is partial.  x and the packed
+    stream sit at the front of larger buffers whose remainder is filled with 0x7F bytes (fp16 NaN
+    patterns behind x): results equal the oracle and do not change with what follows the operands."""
+    from qtip_amd import ops
+    L = make_layer(m, k, K, seed=11 * m + k + K)
+    ref = c_oracle.matvec(L["packed"], L["x"].reshape(-1), L["tlut"], m, k, K)
+    tl = dev(L["tlut"])
+    pk_np = L["packed"].reshape(-1).view(np.uint8)
+    x_np = L["x"].reshape(-1).view(np.uint8)
+    outs = []
+    for fill in (0x7F, 0x00):
+        big_pk = torch.full((pk_np.size + 8192,), fill, dtype=torch.uint8, device="cuda")
+        big_pk[:pk_np.size] = dev(pk_np)
+        big_x = torch.full((x_np.size + 4096,), fill, dtype=torch.uint8, device="cuda")
+        big_x[:x_np.size] = dev(x_np)
+        pk = big_pk[:pk_np.size].view(torch.int16)
+        x = big_x[:x_np.size].view(torch.float16)
+        out = ops.decompress_matvec(pk, x, tl, m, k, K, split_k=False)
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()
+        assert_close(got, ref)
+        outs.append(out)
+        if m <= 512:
+            # batched kernels on the same operands (the activations of the missing columns are zero-filled)
+            X = torch.randn(8, k, generator=torch.Generator().manual_seed(k)).half()
+            big_X = torch.full((X.numel() * 2 + 4096,), fill, dtype=torch.uint8, device="cuda")
+            big_X[:X.numel() * 2] = X.view(torch.uint8).reshape(-1).cuda()
+            gb = ops.decompress_gemm(pk, big_X[:X.numel() * 2].view(torch.float16).view(8, k), tl, m, k, K, round_f16=False)
+            W = c_oracle.decode(L["packed"], L["tlut"], m, k, K).astype(np.float64)
+            assert np.isfinite(gb.cpu().numpy()).all()
+            assert_close(gb.cpu().numpy(), X.double().numpy() @ W.T)
+            outs.append(gb)
+    half = len(outs) // 2
+    for a, b in zip(outs[:half], outs[half:]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("m,k,K", MATVEC_CASES)
 def test_matrix_at_full_size(m, k, K):
     """decode bit-exact; matvec with and without the k split, as partial vectors, through the

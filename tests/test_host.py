@@ -45,6 +45,19 @@ def test_measurement_aids_live_in_a_library_of_their_own():
         assert not hasattr(main, name), name
 
 
+def test_python_host_never_routes_through_the_shared_scratch_entry_point():
+    """qtip_decompress_matvec_noalloc keeps its partial sums in one array per GPU, so overlapping
+    calls race: it is for callers of the C ABI that accept that.  The package's own wrappers (which
+    serve any number of streams) bind it but never call it."""
+    import glob
+    hits = []
+    for path in glob.glob(os.path.join(ROOT, "qtip_amd", "**", "*.py"), recursive=True):
+        for n, line in enumerate(open(path), 1):
+            if "qtip_decompress_matvec_noalloc" in line and not path.endswith("_lib.py"):
+                hits.append((path, n))
+    assert hits == []
+
+
 def test_argument_rejection_without_gpu():
     # rejected arguments return a negative code before anything touches the device
     from qtip_amd import _lib
@@ -153,6 +166,36 @@ def test_get_hadK_and_bits():
         for j in range(20):
             b = j * 20 + i
             assert ((w[b >> 5] >> (b & 31)) & 1) == neg[i, j]
+
+
+def test_had_bits_cache_follows_the_memory_not_the_object():
+    """A caller's own table: a fresh view of the same memory hits the cache (no repacking, hence no
+    device-to-host copy per forward), an in-place change or a new tensor misses, and an entry
+    disappears with the storage it was packed from."""
+    import gc
+    from qtip_amd.utils import matmul_had as mh
+    rng = np.random.default_rng(3)
+    K = 8  # no built-in table of this order: the caller's own entry is used
+    h = torch.from_numpy(np.where(rng.integers(0, 2, (K, K)) > 0, 1.0, -1.0).astype(np.float32))
+    mh._bit_cache.clear()
+    b0 = mh.had_bits(h, K, False, "cpu")
+    n_entries = len(mh._bit_cache)
+    assert mh.had_bits(h.data, K, False, "cpu") is b0          # another tensor object, same memory
+    assert mh.had_bits(h.view(K, K), K, False, "cpu") is b0
+    assert len(mh._bit_cache) == n_entries
+    bt = mh.had_bits(h, K, True, "cpu")
+    assert bt is not b0 and torch.equal(bt, torch.from_numpy(mh._pack_bits((h.numpy() < 0).T)))
+    h[0, 0] = -h[0, 0]                                          # in-place edit: version bump, repacked
+    b1 = mh.had_bits(h, K, False, "cpu")
+    assert b1 is not b0 and torch.equal(b1, torch.from_numpy(mh._pack_bits(h.numpy() < 0)))
+    h2 = h.clone()
+    assert mh.had_bits(h2, K, False, "cpu") is not b1           # other memory: its own entry
+    before = len(mh._bit_cache)
+    del h2
+    gc.collect()
+    assert len(mh._bit_cache) == before - 1                     # freed storage: entry dropped
+    with pytest.raises(ValueError):
+        mh.had_bits(torch.zeros(K, K), K, False, "cpu")
 
 
 def test_quantiser_entry_points_raise():
