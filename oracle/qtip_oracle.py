@@ -385,15 +385,16 @@ def bitshift_linear_forward(inp, packed, SU, SV, tlut, K, return_parts=False, ma
     return out
 
 
-def dense_equivalent(packed, SU, SV, tlut, K):
+def dense_equivalent(packed, SU, SV, tlut, K, decode_fn=None):
     """W_eff with out = inp @ W_eff^T (no activation rounding), following the
     reference's own dense form (lib/codebook/bitshift.py:389-413 and
     quantize_llama/manifest_model.py:38-50):
-    W_eff = diag(SV*32) . H_R . (hatW/32) . H_L^T . diag(SU)."""
+    W_eff = diag(SV*32) . H_R . (hatW/32) . H_L^T . diag(SU).
+    decode_fn(packed, tlut, m, n, K): a faster restatement of decode_kernel (the C one)."""
     SU = np.asarray(SU, dtype=np.float64)
     SV = np.asarray(SV, dtype=np.float64)
     n, m = SU.shape[0], SV.shape[0]
-    w = decode_kernel(packed, tlut, m, n, K).astype(np.float64) / 32.0
+    w = (decode_fn or decode_kernel)(packed, tlut, m, n, K).astype(np.float64) / 32.0
     # rows of w are vectors over n: apply H_L (not transposed) to each row,
     # since (w H_L^T)[i,:] = H_L-transform of row i with the transposed table
     # swapped: (w @ HL^T) = (HL @ w^T)^T

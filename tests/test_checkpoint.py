@@ -203,6 +203,51 @@ def test_untied_checkpoint_without_lm_head_is_incomplete(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tie", [False, True])
+def test_reference_schema_checkpoint_on_the_gpu_runs_like_its_dense_model(tmp_path, tie):
+    """The reference-keyed checkpoint loaded onto the GPU: the logits of the loaded model (module
+    path over a prompt, then the fused decode step) against a float64 dense model assembled from the
+    checkpoint's own tensors by key - a tensor the loader put in the wrong place changes them."""
+    import numpy as np
+    import decoder_ref
+    from oracle import c_oracle
+    from oracle import qtip_oracle as O
+    ex, tensors = _reference_schema_checkpoint(tmp_path, tie)
+    dev = torch.device('cuda:0')
+    model = C.load_llama(str(tmp_path), max_cache_len=32, device=dev)
+    assert model.embed.is_cuda and model.layers[0].q_proj.trellis.is_cuda
+    f64 = lambda k: tensors[k].numpy().astype(np.float64)
+
+    def dense(prefix):
+        if prefix + '.weight' in tensors:
+            return f64(prefix + '.weight')
+        g = lambda leaf: tensors[prefix + '.' + leaf].numpy()
+        return O.dense_equivalent(g('trellis'), g('SU'), g('SV'), g('tlut'), 2, decode_fn=c_oracle.decode)
+
+    layers = []
+    for i in range(ex['num_hidden_layers']):
+        a, m = f'model.layers.{i}.self_attn.', f'model.layers.{i}.mlp.'
+        layers.append({"in_norm": f64(f'model.layers.{i}.input_layernorm.weight'),
+                       "post_norm": f64(f'model.layers.{i}.post_attention_layernorm.weight'),
+                       "q": dense(a + 'q_proj'), "k": dense(a + 'k_proj'), "v": dense(a + 'v_proj'), "o": dense(a + 'o_proj'),
+                       "gate": dense(m + 'gate_proj'), "up": dense(m + 'up_proj'), "down": dense(m + 'down_proj')})
+    W = {"embed": f64('model.embed_tokens.weight'), "norm": f64('model.norm.weight'), "layers": layers,
+         "lm_head": f64('model.embed_tokens.weight' if tie else 'lm_head.weight')}
+    ids = torch.randint(0, 96, (8,), generator=torch.Generator().manual_seed(2))
+    ref, _ = decoder_ref.forward(W, model.cfg, ids.numpy())
+
+    def close(got, want):
+        d = np.abs(got.astype(np.float64) - want)
+        assert d.max() <= 2e-2 * np.abs(want).max() and d.mean() <= 5e-3 * np.abs(want).mean()
+
+    with torch.no_grad():
+        lg = model(ids[None, :7].to(dev), torch.arange(7, device=dev))
+        close(lg[0].cpu().numpy(), ref[:7])
+        got = model.decode_fused(ids[7].view(1, 1).to(dev), torch.tensor([7], device=dev))
+        close(got[0, 0].cpu().numpy(), ref[7])
+
+
+@pytest.mark.gpu
 def test_loaded_model_runs_like_the_original(tmp_path):
     from qtip_amd.llama_decode import generate
     dev = torch.device('cuda:0')

@@ -56,6 +56,46 @@ def test_first_call_inside_a_capture_is_a_defined_error_then_init_and_capture_wo
     assert res.returncode == 0 and "ok" in res.stdout, res.stdout + res.stderr
 
 
+def test_size_queries_as_first_call_inside_a_capture_run_no_set_up():
+    """The size queries may be a process's first library call and may come during a capture: they
+    answer from the CU count alone (no hipFuncSetAttribute inside the capture), the capture stays
+    valid, and the device still counts as not set up for a launcher in the same capture."""
+    code = textwrap.dedent("""
+        import ctypes, sys
+        import torch
+        sys.path.insert(0, %r)
+        from qtip_amd._lib import LIB_PATH
+        lb = ctypes.CDLL(LIB_PATH)
+        lb.qtip_matvec_workspace_bytes.restype = ctypes.c_size_t
+        lb.qtip_gemm_workspace_bytes.restype = ctypes.c_size_t
+        lb.qtip_decompress_matvec.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        m, k, K = 128, 28672, 2
+        g = torch.Generator().manual_seed(0)
+        pk = torch.randint(-32768, 32768, (m * k * K // 16,), dtype=torch.int16, generator=g).cuda()
+        tl = torch.randn(512, 2, generator=g).half().cuda()
+        x = torch.randn(k, generator=g).half().cuda()
+        out = torch.zeros(m, device="cuda")
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            split = lb.qtip_matvec_split(m, k, K)
+            need = lb.qtip_matvec_workspace_bytes(m, k, K)
+            gneed = lb.qtip_gemm_workspace_bytes(m, k, K, 8)
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = lb.qtip_decompress_matvec(out.data_ptr(), pk.data_ptr(), x.data_ptr(), tl.data_ptr(), m, k, K, None, 0, st)
+            y = x * 2
+        assert split > 1 and need > 0 and need %% (m * 4) == 0 and gneed > 0, (split, need, gneed)
+        assert rc == -7, rc
+        graph.replay(); torch.cuda.synchronize()
+        assert torch.equal(y, x * 2)
+        assert lb.qtip_init() == 0
+        assert lb.qtip_matvec_split(m, k, K) == split and lb.qtip_matvec_workspace_bytes(m, k, K) == need
+        print("ok")
+    """) % ROOT
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and "ok" in res.stdout, res.stdout + res.stderr
+
+
 def test_workspace_growth_keeps_the_buffer_a_recorded_graph_writes_to():
     """A graph recorded with the split-k workspace of the moment keeps working after a later,
     larger request replaced that workspace: the old buffer stays allocated."""

@@ -948,10 +948,22 @@ def test_fused_decode_with_per_shard_transforms(fused):
         l0.__dict__.pop(name, None)
     out_g, _, _ = generate(model, ids, 6, use_graph=True, fused=True)
     out_e, _, _ = generate(model, ids, 6, use_graph=False, fused=True)
-    out_m, _, _ = generate(model, ids, 6, use_graph=False, fused=False)
-    assert torch.equal(out_g, out_e)
-    assert out_g.shape == (1, 6) and out_m.shape == (1, 6)
-    assert int(out_g[0, 0]) == int(out_m[0, 0])  # the prompt's pick; later greedy picks may part on a near-tie
+    assert torch.equal(out_g, out_e) and out_g.shape == (1, 6)
+    # the steps after the first, teacher-forced: the tokens the fused loop decoded go through the
+    # module path and through the fused step position by position (greedy picks of two paths may
+    # part on a near-tie, logits and caches may not differ by more than the rounding allows)
+    with torch.no_grad():
+        model(ids, torch.arange(9, device="cuda"))
+        for t in range(5):
+            tok, pos = out_g[:, t:t + 1].contiguous(), torch.tensor([9 + t], device="cuda")
+            a = model(tok, pos)
+            kc = [c.clone() for c in model.k_cache + model.v_cache]
+            for c in model.k_cache + model.v_cache:
+                c[:, :, 9 + t].zero_()
+            b = model.decode_fused(tok, pos)
+            assert_close(b.cpu().numpy(), a.cpu().numpy(), 2e-2, 5e-3)
+            for c0, c1 in zip(kc, model.k_cache + model.v_cache):
+                assert torch.allclose(c0[:, :, :10 + t].float(), c1[:, :, :10 + t].float(), atol=2e-2)
 
 
 def test_sample_pick_draws_from_the_reference_distribution():
@@ -1143,8 +1155,6 @@ def test_grouped_matvec_with_layer_boundary(K, ms, k, S, Sp):
     single-matrix launch bit for bit (a row block is summed by one workgroup in a fixed order,
     whichever workgroup that is)."""
     from qtip_amd import ops
-    if K != 2 and sum(ms) > 12288:
-        pytest.skip("large shapes once")
     g = torch.Generator().manual_seed(K + sum(ms) + Sp)
     layers = [make_layer(m, k, K, seed=m + k + K + i) for i, m in enumerate(ms)]
     prev = torch.randn(Sp, 1, k, generator=g).cuda()
@@ -1174,8 +1184,6 @@ def test_grouped_plain_matvec(K, ms, k, S):
     """Up to three matrices, each on its own input, in one launch: bit-identical to the
     single-matrix launches."""
     from qtip_amd import ops
-    if K != 2 and sum(ms) > 16384:
-        pytest.skip("large shapes once")
     layers = [make_layer(m, k, K, seed=m + k + K + 7 * i) for i, m in enumerate(ms)]
     packed = [dev(L["packed"]).reshape(-1) for L in layers]
     tluts = [dev(L["tlut"]).reshape(-1) for L in layers]

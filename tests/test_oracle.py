@@ -277,3 +277,21 @@ def test_layer_linearity_in_SV():
     _, p1 = O.bitshift_linear_forward(L["x"], L["packed"], L["SU"], L["SV"], L["tlut"], 2, return_parts=True)
     _, p2 = O.bitshift_linear_forward(L["x"], L["packed"], L["SU"], 2 * L["SV"], L["tlut"], 2, return_parts=True)
     np.testing.assert_allclose(p2["y2"], 2 * p1["y2"], rtol=1e-12)
+
+
+def test_cpu_baseline_path_decodes_like_the_c_oracle():
+    """oracle/torch_cpu_path.py (the code bench.py times as cpu_baseline) against the C
+    restatement of the decode, bit for bit, and its matvec against the C matvec."""
+    import torch
+    from oracle import c_oracle, torch_cpu_path
+    from synth import make_layer
+    for (m, k, K) in [(64, 96, 2), (32, 256, 3), (128, 64, 4), (256, 1024 + 32, 2)]:
+        L = make_layer(m, k, K, seed=m + k + K)
+        lut = torch_cpu_path.expand_lut(torch.from_numpy(L["tlut"]))
+        w = torch_cpu_path.decode_dense(torch.from_numpy(L["packed"]), lut, m, k, K).numpy()
+        ref = c_oracle.decode(L["packed"], L["tlut"], m, k, K)
+        assert np.array_equal(w.view(np.uint16), ref.view(np.uint16)), (m, k, K)
+        r = torch_cpu_path.time_layer(torch.from_numpy(L["packed"]), torch.from_numpy(L["x"]), torch.from_numpy(L["tlut"]),
+                                      m, k, K)
+        want = c_oracle.matvec(L["packed"], L["x"].reshape(-1), L["tlut"], m, k, K)
+        assert np.abs(r["out"].numpy() - want).max() <= 1e-4 * np.abs(want).max()
