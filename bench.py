@@ -64,6 +64,48 @@ def measured_traffic(workload, bits):
         os.path.relpath(TRAFFIC_FILE, ROOT)
 
 
+def timeline(shapes, ms_per_step):
+    """In-kernel readings of the 100 MHz constant clock kept by the timeline build (see QTIP_STAMPS in
+    qtip_amd/csrc/qtip_hip.hip): after the timed graph replay the buffer holds, per shape, the last
+    launch of that shape - i.e. the last step.  All figures in microseconds (10 ns resolution)."""
+    import ctypes
+    import numpy as np
+    from qtip_amd import _lib
+    L = _lib.lib()
+    if not hasattr(L, "qtip_debug_stamps"):
+        raise RuntimeError("--timeline needs the library built with -DQTIP_STAMPS (python -m bench_probe)")
+    buf = np.zeros(64 * 256 * 16, dtype=np.uint64)
+    L.qtip_debug_stamps.argtypes = [ctypes.c_void_p]
+    rc = L.qtip_debug_stamps(buf.ctypes.data)
+    if rc != 0:
+        raise RuntimeError(f"qtip_debug_stamps failed ({rc})")
+    st = buf.reshape(64, 256, 16).astype(np.int64)
+    us = lambda ticks: round(float(ticks) / 100.0, 2)
+    fml = lambda a: [us(a.min()), us(np.median(a)), us(a.max())]
+    rows, ends, prev_end = {}, [], None
+    for name, m, k in shapes:
+        s = st[((m ^ k) >> 10) & 63]
+        s = s[s[:, 0] > 0]
+        t0 = s[:, 0].min()
+        row = {"workgroups": int(len(s)),
+               "previous_launch_last_end_to_first_start": us(t0 - prev_end) if prev_end is not None else None,
+               "workgroup_starts_first_median_last": fml(s[:, 0] - t0),
+               "wave15_start_after_wave0": fml(s[:, 5] - s[:, 0]),
+               "start_to_table_words_picked": fml(s[:, 1] - s[:, 0]),
+               "start_to_first_barrier_reached": fml(s[:, 2] - s[:, 0]),
+               "start_to_first_barrier_passed": fml(s[:, 3] - s[:, 0]),
+               "start_to_first_weights_in_registers": fml(s[:, 15] - s[:, 0]),
+               "workgroup_ends_first_median_last_from_first_start": fml(s[:, 4] - t0),
+               "span_first_start_to_last_end": us(s[:, 4].max() - t0)}
+        prev_end = s[:, 4].max()
+        ends.append((t0, prev_end))
+        rows[name] = row
+    spans = sum(e - b for b, e in ends)
+    return {"clock": "s_memrealtime, 100 MHz", "launches_of_the_last_step": rows,
+            "sum_of_spans_us": us(spans), "first_start_to_last_end_us": us(ends[-1][1] - ends[0][0]),
+            "ms_per_step_of_this_run": round(ms_per_step, 5)}
+
+
 SHAPES_70B = [("qkv", 10240, 8192), ("o", 8192, 8192), ("up_gate", 57344, 8192), ("down", 8192, 28672)]
 SHAPES_7B = [("qkv", 12288, 4096), ("o", 4096, 4096), ("up_gate", 22016, 4096), ("down", 4096, 11008)]
 
@@ -94,6 +136,11 @@ def main():
                          "ceilings, e2e, e2e13b, e2e70b (counter runs under rocprofv3 pick one)")
     ap.add_argument("--print-kernel-source-digest", action="store_true",
                     help="print the digest that profiles/matvec_k2_llama70b_set_traffic.txt must name, and exit")
+    ap.add_argument("--timeline", action="store_true",
+                    help="run on the timeline build of the library (bench_probe/libqtip_hip_stamped.so: the product "
+                         "sources compiled with -DQTIP_STAMPS, `python -m bench_probe`) and add the in-kernel clock "
+                         "readings of the last timed step to the line: per launch, previous end -> first start, "
+                         "start -> first barrier, first / median / last workgroup end")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs)")
@@ -106,6 +153,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.timeline:
+        import bench_probe
+        os.environ["QTIP_HIP_LIBRARY"] = bench_probe.STAMPED_LIB_PATH
     import torch
     from qtip_amd import ops
 
@@ -239,6 +289,9 @@ def main():
         },
         "host_wall_s_timed_region": round(wall_s, 4),
     }
+
+    if args.timeline:
+        result["timeline"] = timeline(shapes, ms_per_step)
 
     # ---- per-shape kernel times and whole-layer times ---------------------
     extras = set() if args.no_extras else set(args.extras.split(","))

@@ -12,6 +12,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libqtip_probe.so")
 SRC = os.path.join(HERE, "qtip_probe.hip")
 
+# the product sources compiled with -DQTIP_STAMPS: wave 0 of every matvec workgroup records a few
+# readings of the constant clock (bench.py --timeline prints them); never loaded by default
+STAMPED_LIB_PATH = os.path.join(HERE, "libqtip_hip_stamped.so")
+
 OPS_PER_ITER = 88
 KINDS = {"v_and_b32": 0, "v_add_u32": 1, "v_lshrrev_b32": 2, "v_lshlrev_b32": 3, "v_pk_mad_u16": 4,
          "v_mad_u32_u16": 5, "v_perm_b32": 6, "v_pk_lshrrev_b16": 7, "v_mov_b32_dpp": 8, "v_dot2c_f32_f16": 9,
@@ -38,6 +42,20 @@ def build(verbose=True):
         print(err, file=sys.stderr)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     return LIB_PATH
+
+
+def build_stamped(verbose=True):
+    """The timeline build of libqtip_hip.so (same sources and flags, plus -DQTIP_STAMPS)."""
+    from qtip_amd import build as qbuild
+    cmd = [os.environ.get("HIPCC", "hipcc")] + qbuild.HIPCC_FLAGS + ["-DQTIP_STAMPS"] + qbuild.SRCS + \
+        ["-o", STAMPED_LIB_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
+    os.replace(STAMPED_LIB_PATH + ".tmp", STAMPED_LIB_PATH)
+    return STAMPED_LIB_PATH
 
 
 def lib():

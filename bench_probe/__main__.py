@@ -1,3 +1,4 @@
-from . import build
+from . import build, build_stamped
 
 build()
+build_stamped()

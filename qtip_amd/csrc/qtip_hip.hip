@@ -239,6 +239,26 @@ struct GroupArgs {
   int upw_q[3], upw_r[3];
   size_t part_stride;         // floats between partial results
 };
+// Timeline build (-DQTIP_STAMPS, used by `bench.py --timeline` through a library of its own; the
+// product library is built without it): waves 0 and 15 of every matvec workgroup keep a few
+// readings of the 100 MHz constant clock in registers and wave 0 stores them when it ends, into
+// the slot of its launch's shape, so that after a graph replay the buffer holds the last launch
+// of every shape.
+//   0 first instruction   1 table words picked   2 at the first barrier   3 past it
+//   4 end of the kernel   5 first instruction of wave 15   15 first wave-load of wave 0 in registers
+// (nothing is read inside the loop: a clock reading there makes every wait in it a full one; and
+// only two waves read the clock: 4096 waves reading it at once queue up behind each other)
+#ifdef QTIP_STAMPS
+constexpr int kStampSlots = 64, kStampWgs = 256, kStampN = 16;
+__device__ unsigned long long g_stamps[kStampSlots][kStampWgs][kStampN];
+#define QTIP_STAMP_DECL unsigned long long stamp_v[kStampN] = {};
+#define QTIP_STAMP(i) if (wave == 0 || (i == 0 && wave == kWaves - 1)) stamp_v[i] = __builtin_amdgcn_s_memrealtime();
+#define QTIP_STAMP_FIRST_LOAD() if (wave == 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DEPTH - 1)); stamp_v[15] = __builtin_amdgcn_s_memrealtime(); }
+#else
+#define QTIP_STAMP_DECL
+#define QTIP_STAMP(i)
+#define QTIP_STAMP_FIRST_LOAD()
+#endif
 template <typename T>
 __device__ __forceinline__ T pick3(const T (&a)[3], int g) {
   return g == 0 ? a[0] : (g == 1 ? a[1] : a[2]);
@@ -389,6 +409,8 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
   uint8_t* xs_lds = smem + kLut128Bytes + 2 * kWaves * 32 * sizeof(float);  // [wl_per][256] when XLDS
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  QTIP_STAMP_DECL
+  QTIP_STAMP(0)
   const int a = lane & 15, g = lane >> 4;
   const uint32_t slot4 = lds_address(lut) + ((uint32_t)(lane & 31) << 2);
   const int nkb = k >> 5;
@@ -475,6 +497,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     for (int j = 1; j < 8; ++j) v = ((lane >> 3) == j) ? sw[j] : v;
     tw[it] = v;
   }
+  QTIP_STAMP(1)
   u32x4 xstage[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
   u32x4 xstage2[XHALF ? 2 : 1] = {};
   const int jh = XHALF ? (npw + 1) >> 1 : npw;  // items per wave served by the first staging
@@ -559,9 +582,12 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       if (o < xbytes) *reinterpret_cast<u32x4*>(xs_lds + o) = xstage[ps];
     }
   }
+  QTIP_STAMP(2)
   __syncthreads();
+  QTIP_STAMP(3)
 #pragma unroll
   for (int d = FIRST; d < DEPTH; ++d) issue(d);
+  QTIP_STAMP_FIRST_LOAD()
 
   // wave-load w_first (the transformed vector is stored whole, a staged one from wl0 on)
   const uint32_t xs_lane = lds_address(xs_lds) + xoff + (uint32_t)(XFORM ? w_first : wave) * 256u;
@@ -671,6 +697,22 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       else run(std::integral_constant<int, 0>{}, T_full, T);
     }
   }
+#ifdef QTIP_STAMPS
+  {
+    QTIP_STAMP(4)
+    const int wg = (int)blockIdx.x + (int)gridDim.x * (int)blockIdx.y;
+    const int slot = ((m ^ k) >> 10) & (kStampSlots - 1);
+    if (wg < kStampWgs && lane == 0) {
+      if (wave == 0) {
+#pragma unroll
+        for (int i = 0; i < kStampN; ++i)
+          if (i != 5) g_stamps[slot][wg][i] = stamp_v[i];
+      } else if (wave == kWaves - 1) {
+        g_stamps[slot][wg][5] = stamp_v[0];
+      }
+    }
+  }
+#endif
 }
 
 // out[i] = parts[0][i] + parts[1][i] + ... in that order
@@ -1582,6 +1624,16 @@ static int check_matvec(const void* out, const void* packed, const void* x_f16, 
     return QTIP_E_ALIGN;
   return QTIP_OK;
 }
+
+#ifdef QTIP_STAMPS
+// copies the clock readings of the timeline build (64 x 256 x 16 x 8 bytes) to host memory;
+// synchronises the device
+int qtip_debug_stamps(void* host_buf) {
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpyFromSymbol(host_buf, HIP_SYMBOL(g_stamps), sizeof(g_stamps));
+  return (int)e;
+}
+#endif
 
 int qtip_decompress_matvec_parts(float* parts, const void* packed, const void* x_f16,
                                  const void* tlut, int m, int k, int bits, int nparts,
