@@ -141,6 +141,10 @@ def main():
                          "sources compiled with -DQTIP_STAMPS, `python -m bench_probe`) and add the in-kernel clock "
                          "readings of the last timed step to the line: per launch, previous end -> first start, "
                          "start -> first barrier, first / median / last workgroup end")
+    ap.add_argument("--calibrate-probe", action="store_true",
+                    help="also time 64 launches of the stream-read probe on a fixed 64 MiB buffer in one graph (a kernel "
+                         "of known duration: run once plain and once under rocprofv3 --kernel-trace, the difference "
+                         "between the trace's mean for it and the plain figure is what the profiler adds per launch)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs)")
@@ -292,6 +296,13 @@ def main():
 
     if args.timeline:
         result["timeline"] = timeline(shapes, ms_per_step)
+    if args.calibrate_probe:
+        import bench_probe
+        psrc = torch.empty(64 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        gr = capture(lambda: [bench_probe.stream_read(psrc) for _ in range(64)])
+        result["probe_calibration"] = {"kernel": "stream_read_probe_kernel", "bytes": psrc.numel(), "launches": 64,
+                                       "us_per_launch": round(timed(gr, 3, args.settle_ms / 3) * 1e6 / 64, 3)}
+        del gr, psrc
 
     # ---- per-shape kernel times and whole-layer times ---------------------
     extras = set() if args.no_extras else set(args.extras.split(","))
