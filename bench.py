@@ -64,7 +64,7 @@ def measured_traffic(workload, bits):
         os.path.relpath(TRAFFIC_FILE, ROOT)
 
 
-def timeline(shapes, ms_per_step):
+def timeline(shapes, ms_per_step, chained=False):
     """In-kernel readings of the 100 MHz constant clock kept by the timeline build (see QTIP_STAMPS in
     qtip_amd/csrc/qtip_hip.hip): after the timed graph replay the buffer holds, per shape, the last
     launch of that shape - i.e. the last step.  All figures in microseconds (10 ns resolution)."""
@@ -97,10 +97,19 @@ def timeline(shapes, ms_per_step):
                "start_to_first_weights_in_registers": fml(s[:, 15] - s[:, 0]),
                "workgroup_ends_first_median_last_from_first_start": fml(s[:, 4] - t0),
                "span_first_start_to_last_end": us(s[:, 4].max() - t0)}
+        if chained and (s[:, 10] > 0).all():
+            # the transform / layer boundary in the prologue (wave 0): entered, past its three barriers, left
+            row["prologue_transform_entered_barriers_left"] = [fml(s[:, i] - s[:, 0])[1] for i in (6, 7, 8, 9, 10)
+                                                               if (s[:, i] > 0).all()]
+        if chained:
+            row["previous_launch_last_end_to_first_start"] = None  # other kernels run between these launches
         prev_end = s[:, 4].max()
         ends.append((t0, prev_end))
         rows[name] = row
     spans = sum(e - b for b, e in ends)
+    if chained:
+        return {"clock": "s_memrealtime, 100 MHz", "matvec_launches_of_the_last_layer": rows,
+                "sum_of_spans_us": us(spans), "first_start_to_last_end_us": us(ends[-1][1] - ends[0][0])}
     return {"clock": "s_memrealtime, 100 MHz", "launches_of_the_last_step": rows,
             "sum_of_spans_us": us(spans), "first_start_to_last_end_us": us(ends[-1][1] - ends[0][0]),
             "ms_per_step_of_this_run": round(ms_per_step, 5)}
@@ -494,6 +503,10 @@ def main():
                                 "ms_per_token": round(1e3 / tps, 3), "distinct_new_tokens": _distinct(toks, 256),
                                 "bytes_per_token": tok_bytes,
                                 "frac_hbm": round(tok_bytes * tps / 1e9 / HBM_PEAK_GBS, 4)}
+        if args.timeline:
+            # the four matvec launches of the last layer of the last decoded token (qkv and up/gate with the
+            # layer boundary in their prologue, o with its input transform, down plain)
+            result["e2e_decode"]["timeline"] = timeline(SHAPES_7B, 1e3 / tps, chained=True)
         del model
         torch.cuda.empty_cache()
         # the layout of the published checkpoints: seven separate projections per layer (grouped launches)

@@ -246,6 +246,7 @@ struct GroupArgs {
 // of every shape.
 //   0 first instruction   1 table words picked   2 at the first barrier   3 past it
 //   4 end of the kernel   5 first instruction of wave 15   15 first wave-load of wave 0 in registers
+//   6-10 the transform / layer boundary of the prologue (see QTIP_STAMP_SV)
 // (nothing is read inside the loop: a clock reading there makes every wait in it a full one; and
 // only two waves read the clock: 4096 waves reading it at once queue up behind each other)
 #ifdef QTIP_STAMPS
@@ -254,10 +255,16 @@ __device__ unsigned long long g_stamps[kStampSlots][kStampWgs][kStampN];
 #define QTIP_STAMP_DECL unsigned long long stamp_v[kStampN] = {};
 #define QTIP_STAMP(i) if (wave == 0 || (i == 0 && wave == kWaves - 1)) stamp_v[i] = __builtin_amdgcn_s_memrealtime();
 #define QTIP_STAMP_FIRST_LOAD() if (wave == 0) { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DEPTH - 1)); stamp_v[15] = __builtin_amdgcn_s_memrealtime(); }
+// inside the layer boundary of the prologue (sv = the kernel's stamp_v): 6 entered, 7 / 8 / 9 past its
+// first / second / third barrier (first transform, RMSNorm sum, second transform), 10 left
+#define QTIP_STAMP_SV(i) if (wave == 0 && sv) sv[i] = __builtin_amdgcn_s_memrealtime();
+#define QTIP_STAMP_PTR stamp_v
 #else
 #define QTIP_STAMP_DECL
 #define QTIP_STAMP(i)
 #define QTIP_STAMP_FIRST_LOAD()
+#define QTIP_STAMP_SV(i)
+#define QTIP_STAMP_PTR nullptr
 #endif
 template <typename T>
 __device__ __forceinline__ T pick3(const T (&a)[3], int g) {
@@ -292,9 +299,11 @@ __device__ __forceinline__ void chain_load(const ChainArgs& c, const _Float16* s
 template <int EPT>
 __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, float scale_in, float* xbuf,
                                               float* wsum, _Float16* xs, int tid, int lane, int wave,
-                                              bool write_x) {
+                                              bool write_x, unsigned long long* sv = nullptr) {
   using namespace qtip_wht;
   constexpr int N = kThreads * EPT;
+  (void)sv;
+  QTIP_STAMP_SV(6)
   const int e_nat = tid * EPT;
   const int e_swp = (((lane & 15) << 6) | ((wave & 15) << 2) | (lane >> 4)) * EPT;
   float v[EPT];
@@ -307,6 +316,7 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 #pragma unroll
   for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_nat + i)] = v[i];
   __syncthreads();
+  QTIP_STAMP_SV(7)
 #pragma unroll
   for (int i = 0; i < EPT; ++i) v[i] = wht_lanes(xbuf[xidx<EPT>(e_swp + i)], 4, lane);
   // ---- residual, RMSNorm, sign vector of this layer
@@ -323,6 +333,7 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
   ss = wave_sum(ss);
   if (lane == 0) wsum[wave] = ss;
   __syncthreads();  // also: every read of xbuf above is done
+  QTIP_STAMP_SV(8)
   float tot = 0.f;
 #pragma unroll
   for (int w = 0; w < 16; ++w) tot += wsum[w];
@@ -336,6 +347,7 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
 #pragma unroll
   for (int i = 0; i < EPT; ++i) xbuf[xidx<EPT>(e_swp + i)] = v[i];
   __syncthreads();
+  QTIP_STAMP_SV(9)
   // the bits still missing are the top four of the element's lane field = lane bits 2..5 here
   _Float16 xo[EPT];
 #pragma unroll
@@ -346,6 +358,7 @@ __device__ __forceinline__ void chain_compute(ChainRegs& r, const ChainArgs& c, 
   }
   st_f16<EPT>(xs + e_nat, xo);
   __syncthreads();  // the exchange buffer is free for the table, xs is complete
+  QTIP_STAMP_SV(10)
 }
 
 // Work unit = (32-row block rb, k split s).  The 16 waves of a workgroup take
@@ -555,11 +568,12 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
     _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
     const bool write_x = blockIdx.x == 0 && blockIdx.y == 0;
     switch (k >> 10) {
-      case 2: chain_compute<2>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
-      case 4: chain_compute<4>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
-      default: chain_compute<8>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x); break;
+      case 2: chain_compute<2>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x, QTIP_STAMP_PTR); break;
+      case 4: chain_compute<4>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x, QTIP_STAMP_PTR); break;
+      default: chain_compute<8>(cr, chain, xscale, xbuf, wsum, xs, tid, lane, wave, write_x, QTIP_STAMP_PTR); break;
     }
   } else if constexpr (XFORM == 1) {
+    QTIP_STAMP(6)
     float* xchg = reinterpret_cast<float*>(smem);
     _Float16* xs = reinterpret_cast<_Float16*>(xs_lds);
     switch (k >> 10) {
@@ -567,6 +581,7 @@ __global__ __launch_bounds__(kThreads, 1) void matvec_kernel(
       case 4: xform_prologue<4>(xraw, xscale, xchg, xs, tid, lane, wave); break;
       default: xform_prologue<8>(xraw, xscale, xchg, xs, tid, lane, wave); break;
     }
+    QTIP_STAMP(10)
   }
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
